@@ -1,6 +1,7 @@
 """Typed model configurations read from config.json."""
 
 from .base import ConfigError, ModelConfig, read_config_json
+from .gilozen import GilozenConfig
 from .qwen2 import Qwen2Config
 
-__all__ = ["ConfigError", "ModelConfig", "Qwen2Config", "read_config_json"]
+__all__ = ["ConfigError", "GilozenConfig", "ModelConfig", "Qwen2Config", "read_config_json"]

@@ -36,6 +36,11 @@ class ModelConfig:
     def from_dict(cls, raw: Mapping[str, Any]) -> "ModelConfig":  # pragma: no cover - abstract
         raise NotImplementedError
 
+    def completed_from(self, tensor_shapes: Mapping[str, tuple]) -> "ModelConfig":
+        """The configuration with the sizes that config.json leaves to the checkpoint's tensors filled in
+        from their shapes (name -> shape); most architectures state every size and return themselves."""
+        return self
+
     def to_dict(self) -> dict:  # pragma: no cover - abstract
         """config.json content that ``from_dict`` reads back to an equal configuration."""
         raise NotImplementedError

@@ -55,6 +55,36 @@ int fsie_zero_pages(void* pool_a, void* pool_b, const int32_t* pages, int n, int
 // Counter-based random values (the random-weights mode): see elementwise.hip.
 int fsie_random_fill(void* out, int64_t n, uint64_t key, int kind, float std, hipStream_t stream);
 int fsie_swiglu(const void* x, void* out, int n_tokens, int inter, int dtype, hipStream_t stream);
+// the same with the gate's activation named: 0 = SiLU, 1 = GELU in its tanh form
+int fsie_gated_act(const void* x, void* out, int n_tokens, int inter, int dtype, int act, hipStream_t stream);
+// The norm of a sublayer's output, the residual sum and the next norm in one pass:
+//   v = residual + rmsnorm(delta; post_weight, post_eps);  out = rmsnorm(v; weight, eps)
+// delta as for fsie_rmsnorm (one array of the activations' type, or n_parts float32 partial sums).
+int fsie_sandwich_norm(float* residual, const void* delta, const float* post_weight, float post_eps, const float* weight,
+                       float eps, void* out, const int32_t* rows, int n_rows, int hidden, int dtype, int write_back,
+                       int n_parts, int total_rows, hipStream_t stream);
+// out[t][h][:] = rmsnorm(o[t][h][:]; weight, eps) * act(gate[t][h][:]), o float32, a head `width` values wide
+int fsie_gated_headnorm(const float* o, const void* gate, int64_t gate_stride, const float* weight, void* out, int n_tokens,
+                        int heads, int width, float eps, int act, int dtype, hipStream_t stream);
+// x <- cap * tanh(x / cap) in place
+int fsie_softcap(float* x, int64_t n, float cap, hipStream_t stream);
+
+// Gated linear attention over the tokens of a step, from and to the per-request state (linear_attention.hip).
+int fsie_gla_scan(const void* proj, int64_t proj_stride, int q_off, int k_off, int v_off, const float* z, float* state,
+                  const int32_t* q_starts, const int32_t* seq_slots, int n_seqs, float* out, int heads, int dim, int vdim,
+                  float q_scale, float inv_tau, int n_slots, int dtype, hipStream_t stream);
+
+// Attention through a latent (latent_attention.hip): the norms of the latents, the gates and the cache row of
+// every token; the rotation of pairs of neighbours; a product with a matrix of its own for every head.
+int fsie_latent_prep(const void* proj, int64_t stride, int dq_off, int q_rank, int dkv_off, int kv_rank, int rot_dim,
+                     int rot_pairs, int g_off, int heads, const float* q_weight, const float* kv_weight, float eps,
+                     const float* cos_sin, void* cq, float* gate, const int32_t* slots, void* k_pool, void* v_pool,
+                     int width, int page_size, int64_t pool_slots, int n_tokens, int dtype, hipStream_t stream);
+int fsie_rope_pairs(const void* in, int64_t in_stride, int in_off, int in_hs, void* out, int64_t out_stride, int out_off,
+                    int out_hs, int heads, int width, int rot_pairs, int out_width, const float* cos_sin, int n_tokens,
+                    int dtype, hipStream_t stream);
+int fsie_head_gemm(const void* x, int64_t x_stride, int x_off, int x_hs, const void* w, void* y, int64_t y_stride, int y_off,
+                   int y_hs, const float* gate, int n_tokens, int heads, int N, int K, int dtype, hipStream_t stream);
 int fsie_residual_add(float* residual, const void* delta, int64_t total, int dtype, hipStream_t stream);
 int fsie_bias_add(void* y, const float* bias, int rows, int cols, int dtype, hipStream_t stream);
 
@@ -98,6 +128,9 @@ int fsie_gemm_mfma_wide(const void* x, const void* w, float* y, int M, int N, in
 // the rows of w are gate and up in turn: y is bfloat16 [M, N / 2], silu(gate) * up
 int fsie_gemm_mfma_wide_swiglu(const void* x, const void* w, void* y, int M, int N, int K, int waves, int blocks,
                                int frags, hipStream_t stream);
+// the same with the gate's activation named (0 = SiLU, 1 = GELU in its tanh form)
+int fsie_gemm_mfma_wide_gated(const void* x, const void* w, void* y, int M, int N, int K, int waves, int blocks,
+                              int frags, int act, hipStream_t stream);
 // A bfloat16 matrix [N, K] (K a multiple of 32) copied so that the 64 16-byte units of a block of 16
 // rows and 32 values of K lie together in the order of the lanes that hold them: a wave's load of W
 // is then one piece of 1 KB.  The copy has fsie_fragment_order_size values (N rounded up to 16 rows).
@@ -110,15 +143,18 @@ int fsie_fragment_order(const void* w, void* out, int N, int K, hipStream_t stre
 int fsie_attention_scalar(const void* q, int64_t q_stride, const void* k_pool, const void* v_pool,
                           const int32_t* block_tables, int max_pages, const int32_t* items, int n_items,
                           void* out, float* partials, int n_heads, int n_kv, int head_dim, int page_size,
-                          int window, float scale, int dtype, hipStream_t stream);
+                          int window, float scale, int dtype, const float* sinks, hipStream_t stream);
+// sinks (or null, in every attention entry point that takes it): float32 [n_heads]; exp(sinks[h]) is one more
+// term of the softmax denominator of every query row of head h.  It has no key and no value and is not scaled.
+// Items that leave partial records ignore it; the merge that combines them adds it once.
 int fsie_attention_merge(const float* partials, const int32_t* merges, int n_merges, void* out, int n_heads,
-                         int head_dim, int dtype, hipStream_t stream);
+                         int head_dim, int dtype, const float* sinks, hipStream_t stream);
 int fsie_attention_scalar_tile_tokens(int n_heads, int n_kv);
 
 int fsie_attention_mfma(const void* q, int64_t q_stride, const void* k_pool, const void* v_pool,
                         const int32_t* block_tables, int max_pages, const int32_t* items, int n_items, void* out,
                         float* partials, int n_heads, int n_kv, int head_dim, int page_size, int window, float scale,
-                        int large, int waves, hipStream_t stream);
+                        int large, int waves, const float* sinks, hipStream_t stream);
 // the same for a step of one token a request, from the q/k/v product's partial sums: bias, rotation and the
 // write into the pools happen in the kernel
 int fsie_attention_mfma_qkv_ok(int head_dim, int page_size);
@@ -131,7 +167,7 @@ int fsie_attention_mfma_lds_ok(int head_dim, int page_size);
 int fsie_attention_mfma_lds(const void* q, int64_t q_stride, const void* k_pool, const void* v_pool,
                             const int32_t* block_tables, int max_pages, const int32_t* items, const int32_t* groups,
                             int n_groups, void* out, int n_heads, int n_kv, int head_dim, int page_size, int window,
-                            float scale, hipStream_t stream);
+                            float scale, const float* sinks, hipStream_t stream);
 int fsie_attention_mfma_tiles(int head_dim, int large);
 int fsie_attention_mfma_max_waves(int head_dim);
 

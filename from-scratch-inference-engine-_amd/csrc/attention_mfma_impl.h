@@ -79,6 +79,7 @@ struct QkvSums {
     int64_t part_stride;   // n_tokens * width
     int64_t pool_slots;
     int n_parts, width;
+    const float* sinks;    // [n_heads] or null: exp(sink) joins every row's denominator (any variant)
 };
 
 // Element d of a head after the rotation of the pairs (i, i + HD / 2) by the angles whose
@@ -659,7 +660,9 @@ __global__ __launch_bounds__(QKV && MAXW == 1 ? 256 : 64 * MAXW) __attribute__((
     for (int nt = 0; nt < NT; ++nt) {
         if (!rvalid[nt]) continue;
         if (partial_base < 0) {
-            const float inv = l_tot[nt] > 0.f ? 1.0f / l_tot[nt] : 0.f;
+            float denom = l_tot[nt];
+            if (f.sinks && m_fin[nt] != -INFINITY) denom += __builtin_amdgcn_exp2f(f.sinks[rhead[nt]] * kLog2e - m_fin[nt]);
+            const float inv = denom > 0.f ? 1.0f / denom : 0.f;
             bf16_t* o = out + (static_cast<int64_t>(q_row0 + rtok[nt]) * n_heads + rhead[nt]) * HD + 4 * G;
 #pragma unroll
             for (int dt = 0; dt < HDT; ++dt) {
@@ -687,8 +690,10 @@ __global__ __launch_bounds__(QKV && MAXW == 1 ? 256 : 64 * MAXW) __attribute__((
 template <int HDT, int NT>
 int launch(const void* q, int64_t q_stride, const void* k_pool, const void* v_pool, const int32_t* block_tables,
            int max_pages, const int32_t* items, int n_items, void* out, float* partials, int n_heads, int n_kv,
-           int page_size, int window, float scale, int waves, hipStream_t stream) {
+           int page_size, int window, float scale, int waves, const float* sinks, hipStream_t stream) {
     constexpr int MAXW = NT == 1 ? max_waves<HDT>() : 4;
+    QkvSums only_sinks{};
+    only_sinks.sinks = sinks;
     const int group = n_heads / n_kv;
     const int rows = 16 * NT;
     const int gh = group < rows ? group : rows;
@@ -702,7 +707,7 @@ int launch(const void* q, int64_t q_stride, const void* k_pool, const void* v_po
     attention_mfma_kernel<HDT, NT, W, V><<<grid, THREADS, 0, stream>>>(                                              \
         static_cast<const bf16_t*>(q), q_stride, static_cast<const bf16_t*>(k_pool), static_cast<const bf16_t*>(v_pool), \
         block_tables, max_pages, items, static_cast<bf16_t*>(out), partials, n_heads, n_kv, page_size, window, scale, \
-        gh, head_chunks, QkvSums{})
+        gh, head_chunks, only_sinks)
     const bool v16 = page_size % 8 == 0;
     if (waves == 1) {
         if (v16) FSIE_ATTN_LAUNCH(1, 64, true);
@@ -745,6 +750,6 @@ typedef int (*LaunchQkvFn)(const QkvSums&, const void*, const void*, const int32
                            float*, int, int, int, int, float, int, hipStream_t);
 
 typedef int (*LaunchFn)(const void*, int64_t, const void*, const void*, const int32_t*, int, const int32_t*, int, void*,
-                        float*, int, int, int, int, float, int, hipStream_t);
+                        float*, int, int, int, int, float, int, const float*, hipStream_t);
 
 }  // namespace fsie_attn

@@ -67,7 +67,7 @@ __global__ __launch_bounds__(kLdsThreads) __attribute__((amdgpu_waves_per_eu(HDT
     const bf16_t* __restrict__ v_pool, const int32_t* __restrict__ block_tables, int max_pages,
     const int32_t* __restrict__ items, const int32_t* __restrict__ groups, bf16_t* __restrict__ out, int n_heads,
     int n_kv, int page_size_arg, int window, float scale, int gh, int head_chunks, int n_groups, int n_y,
-    int units_per_die) {
+    int units_per_die, const float* __restrict__ sinks) {
     constexpr int HD = HDT * 16;
     const int page_size = PS > 0 ? PS : page_size_arg;
     constexpr int S32 = HDT / 2;       // 32-wide steps over the head dimension
@@ -402,8 +402,9 @@ __global__ __launch_bounds__(kLdsThreads) __attribute__((amdgpu_waves_per_eu(HDT
     if (!active) return;
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
-        const float l_tot = l_acc[nt][0];
+        float l_tot = l_acc[nt][0];
         if (!rvalid[nt]) continue;
+        if (sinks) l_tot += __builtin_amdgcn_exp2f(fmaf(-m_run[nt], scale2, sinks[rhead[nt]] * kLog2e));
         const float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
         bf16_t* o = out + (static_cast<int64_t>(q_row0 + rtok[nt]) * n_heads + rhead[nt]) * HD + 4 * G;
 #pragma unroll
@@ -419,7 +420,7 @@ __global__ __launch_bounds__(kLdsThreads) __attribute__((amdgpu_waves_per_eu(HDT
 template <int HDT, int PS>
 int launch_lds(const bf16_t* q, int64_t q_stride, const bf16_t* k_pool, const bf16_t* v_pool,
                const int32_t* block_tables, int max_pages, const int32_t* items, const int32_t* groups, int n_groups,
-               bf16_t* out, int n_heads, int n_kv, int page_size, int window, float scale, hipStream_t stream) {
+               bf16_t* out, int n_heads, int n_kv, int page_size, int window, float scale, const float* sinks, hipStream_t stream) {
     const int group = n_heads / n_kv;
     const int gh = group < 32 ? group : 32;
     const int head_chunks = (group + gh - 1) / gh;
@@ -430,7 +431,7 @@ int launch_lds(const bf16_t* q, int64_t q_stride, const bf16_t* k_pool, const bf
     attention_mfma_lds_kernel<HDT, PS><<<grid, kLdsThreads, 0, stream>>>(q, q_stride, k_pool, v_pool, block_tables, max_pages,
                                                                      items, groups, out, n_heads, n_kv, page_size,
                                                                      window, scale, gh, head_chunks, n_groups,
-                                                                     by_die ? ys : 0, max(1, fsie_compute_units() / 8));
+                                                                     by_die ? ys : 0, max(1, fsie_compute_units() / 8), sinks);
     FSIE_CHECK_LAUNCH("attention_mfma_lds");
     return 0;
 }
@@ -451,7 +452,7 @@ extern "C" int fsie_attention_mfma_lds_ok(int head_dim, int page_size) {
 extern "C" int fsie_attention_mfma_lds(const void* q, int64_t q_stride, const void* k_pool, const void* v_pool,
                                        const int32_t* block_tables, int max_pages, const int32_t* items,
                                        const int32_t* groups, int n_groups, void* out, int n_heads, int n_kv,
-                                       int head_dim, int page_size, int window, float scale, hipStream_t stream) {
+                                       int head_dim, int page_size, int window, float scale, const float* sinks, hipStream_t stream) {
     FSIE_REQUIRE(n_groups >= 0 && n_heads > 0 && n_kv > 0 && n_heads % n_kv == 0,
                  "attention_mfma_lds: heads %d must be a positive multiple of kv heads %d", n_heads, n_kv);
     FSIE_REQUIRE(fsie_attention_mfma_lds_ok(head_dim, page_size),
@@ -469,9 +470,9 @@ extern "C" int fsie_attention_mfma_lds(const void* q, int64_t q_stride, const vo
     case H:                                                                                                        \
         return page_size == 16                                                                                     \
                    ? fsie_attn::launch_lds<H, 16>(qq, q_stride, kk, vv, block_tables, max_pages, items, groups,    \
-                                                  n_groups, oo, n_heads, n_kv, page_size, window, scale, stream)   \
+                                                  n_groups, oo, n_heads, n_kv, page_size, window, scale, sinks, stream) \
                    : fsie_attn::launch_lds<H, 0>(qq, q_stride, kk, vv, block_tables, max_pages, items, groups,     \
-                                                 n_groups, oo, n_heads, n_kv, page_size, window, scale, stream)
+                                                 n_groups, oo, n_heads, n_kv, page_size, window, scale, sinks, stream)
     switch (head_dim / 16) {
         FSIE_LDS_CASE(2);
         FSIE_LDS_CASE(4);

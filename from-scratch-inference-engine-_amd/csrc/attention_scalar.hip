@@ -51,7 +51,7 @@ __global__ __launch_bounds__(256) void attention_scalar_kernel(
     const T* __restrict__ q, int64_t q_stride, const T* __restrict__ k_pool, const T* __restrict__ v_pool,
     const int32_t* __restrict__ block_tables, int max_pages, const int32_t* __restrict__ items,
     T* __restrict__ out, float* __restrict__ partials, int n_heads, int n_kv, int hd, int page_size,
-    int window, float scale, int gh, int head_chunks) {
+    int window, float scale, int gh, int head_chunks, const float* __restrict__ sinks) {
     extern __shared__ float lds[];
     float* qs = lds;                          // [kRows][hd]
     float* kv = qs + kRows * hd;              // [kKeys][hd + 1]
@@ -215,7 +215,9 @@ __global__ __launch_bounds__(256) void attention_scalar_kernel(
         if (!(r < n_rows && (r % gh) < gh_here)) continue;
         const int tq = r / gh, hq = h_base + (r % gh);
         if (partial_base < 0) {
-            const float inv = l_run[p] > 0.f ? 1.0f / l_run[p] : 0.f;
+            // a sink is one more term of the denominator, exp(sink) relative to the running maximum; it has no value
+            const float denom = l_run[p] + ((sinks && m_run[p] != -INFINITY) ? expf(sinks[hq] - m_run[p]) : 0.f);
+            const float inv = denom > 0.f ? 1.0f / denom : 0.f;
             T* o = out + (static_cast<int64_t>(q_row0 + tq) * n_heads + hq) * hd;
 #pragma unroll
             for (int i = 0; i < kMaxChunks; ++i) {
@@ -250,7 +252,7 @@ constexpr int kMergeWideFrom = 32;
 template <typename T, int DIMS>
 __global__ __launch_bounds__(256) void attention_merge_kernel(const float* __restrict__ partials,
                                                               const int32_t* __restrict__ merges, T* __restrict__ out,
-                                                              int n_heads, int hd) {
+                                                              int n_heads, int hd, const float* __restrict__ sinks) {
     __shared__ float handed[3][DIMS * 64 + 1];  // of waves 1 to 3: the sums, then the denominator
     const int32_t* mi = merges + static_cast<int64_t>(blockIdx.x) * FSIE_ATTN_MERGE_INTS;
     const int out_row = mi[0], first = mi[1], n_splits = mi[2], stride = mi[3];
@@ -265,6 +267,7 @@ __global__ __launch_bounds__(256) void attention_merge_kernel(const float* __res
     const int64_t rec_step = static_cast<int64_t>(stride) * n_heads * rec_size;
     constexpr int AHEAD = 8;
     float denom = 0.f;  // summed in the order of the splits, as the accumulators are
+    float m_all = -INFINITY;  // the maximum over all splits
     float a[DIMS];
 #pragma unroll
     for (int i = 0; i < DIMS; ++i) a[i] = 0.f;
@@ -283,6 +286,7 @@ __global__ __launch_bounds__(256) void attention_merge_kernel(const float* __res
             for (int i = 0; i < DIMS; ++i) v[j][i] = r[min(lane + 64 * i, hd - 1)];
         }
         const float m = wave_max(lane < n_splits ? ms : -INFINITY);
+        m_all = m;
         const float w = (lane >= n_splits || ms == -INFINITY) ? 0.f : expf(ms - m);
 #pragma unroll
         for (int j = 0; j < AHEAD; ++j) {
@@ -301,6 +305,7 @@ __global__ __launch_bounds__(256) void attention_merge_kernel(const float* __res
             m = fmaxf(m, s < n_splits ? rec0[s * rec_step + hd] : -INFINITY);
         }
         m = wave_max(m);
+        m_all = m;
         // this wave's run of the splits: all of them, or a quarter
         int s_begin = 0, s_end = n_splits;
         if (wide) {
@@ -355,6 +360,7 @@ __global__ __launch_bounds__(256) void attention_merge_kernel(const float* __res
             for (int i = 0; i < DIMS; ++i) a[i] += handed[w][i * 64 + lane];
         }
     }
+    if (sinks && m_all != -INFINITY) denom += expf(sinks[hq] - m_all);  // the sink counts once, after the splits
     const float inv = denom > 0.f ? 1.0f / denom : 0.f;
 #pragma unroll
     for (int i = 0; i < DIMS; ++i) {
@@ -364,12 +370,12 @@ __global__ __launch_bounds__(256) void attention_merge_kernel(const float* __res
 }
 
 template <typename T>
-void launch_merge(const float* partials, const int32_t* merges, int n_merges, T* out, int n_heads, int hd,
+void launch_merge(const float* partials, const int32_t* merges, int n_merges, T* out, int n_heads, int hd, const float* sinks,
                   hipStream_t stream) {
     const dim3 grid(n_merges, n_heads);
-    if (hd <= 64) attention_merge_kernel<T, 1><<<grid, 256, 0, stream>>>(partials, merges, out, n_heads, hd);
-    else if (hd <= 128) attention_merge_kernel<T, 2><<<grid, 256, 0, stream>>>(partials, merges, out, n_heads, hd);
-    else attention_merge_kernel<T, 4><<<grid, 256, 0, stream>>>(partials, merges, out, n_heads, hd);
+    if (hd <= 64) attention_merge_kernel<T, 1><<<grid, 256, 0, stream>>>(partials, merges, out, n_heads, hd, sinks);
+    else if (hd <= 128) attention_merge_kernel<T, 2><<<grid, 256, 0, stream>>>(partials, merges, out, n_heads, hd, sinks);
+    else attention_merge_kernel<T, 4><<<grid, 256, 0, stream>>>(partials, merges, out, n_heads, hd, sinks);
 }
 
 }  // namespace
@@ -378,7 +384,7 @@ extern "C" int fsie_attention_scalar(const void* q, int64_t q_stride, const void
                                      const int32_t* block_tables, int max_pages, const int32_t* items,
                                      int n_items, void* out, float* partials, int n_heads, int n_kv,
                                      int head_dim, int page_size, int window, float scale, int dtype,
-                                     hipStream_t stream) {
+                                     const float* sinks, hipStream_t stream) {
     FSIE_REQUIRE(n_items >= 0 && n_heads > 0 && n_kv > 0 && n_heads % n_kv == 0,
                  "attention: heads %d must be a positive multiple of kv heads %d", n_heads, n_kv);
     FSIE_REQUIRE(head_dim > 0 && head_dim <= 32 * kMaxChunks, "attention: head_dim %d must be in 1..%d",
@@ -398,26 +404,26 @@ extern "C" int fsie_attention_scalar(const void* q, int64_t q_stride, const void
         kernel<<<grid, 256, lds, stream>>>(
             static_cast<const float*>(q), q_stride, static_cast<const float*>(k_pool), static_cast<const float*>(v_pool),
             block_tables, max_pages, items, static_cast<float*>(out), partials, n_heads, n_kv, head_dim, page_size,
-            window, scale, gh, head_chunks);
+            window, scale, gh, head_chunks, sinks);
     } else {
         auto kernel = vec ? attention_scalar_kernel<bf16_t, true> : attention_scalar_kernel<bf16_t, false>;
         kernel<<<grid, 256, lds, stream>>>(
             static_cast<const bf16_t*>(q), q_stride, static_cast<const bf16_t*>(k_pool),
             static_cast<const bf16_t*>(v_pool), block_tables, max_pages, items, static_cast<bf16_t*>(out), partials,
-            n_heads, n_kv, head_dim, page_size, window, scale, gh, head_chunks);
+            n_heads, n_kv, head_dim, page_size, window, scale, gh, head_chunks, sinks);
     }
     FSIE_CHECK_LAUNCH("attention_scalar");
     return 0;
 }
 
 extern "C" int fsie_attention_merge(const float* partials, const int32_t* merges, int n_merges, void* out,
-                                    int n_heads, int head_dim, int dtype, hipStream_t stream) {
+                                    int n_heads, int head_dim, int dtype, const float* sinks, hipStream_t stream) {
     FSIE_REQUIRE(n_merges >= 0 && n_heads > 0 && head_dim > 0, "attention_merge: bad sizes");
     FSIE_REQUIRE(head_dim <= 256, "attention_merge: head_dim %d is larger than 256", head_dim);
     FSIE_REQUIRE(dtype == FSIE_F32 || dtype == FSIE_BF16, "attention_merge: unknown dtype %d", dtype);
     if (n_merges == 0) return 0;
-    if (dtype == FSIE_F32) launch_merge(partials, merges, n_merges, static_cast<float*>(out), n_heads, head_dim, stream);
-    else launch_merge(partials, merges, n_merges, static_cast<bf16_t*>(out), n_heads, head_dim, stream);
+    if (dtype == FSIE_F32) launch_merge(partials, merges, n_merges, static_cast<float*>(out), n_heads, head_dim, sinks, stream);
+    else launch_merge(partials, merges, n_merges, static_cast<bf16_t*>(out), n_heads, head_dim, sinks, stream);
     FSIE_CHECK_LAUNCH("attention_merge");
     return 0;
 }

@@ -262,22 +262,22 @@ void launch_rmsnorm(const NormCall& c) {
 
 // out[t, j] = silu(x[t, 2j]) * x[t, 2j + 1]; x is [T, 2*inter] with gate and up interleaved.
 template <typename T>
-__global__ void swiglu_kernel(const T* __restrict__ x, T* __restrict__ out, int64_t total, int inter) {
+__global__ void swiglu_kernel(const T* __restrict__ x, T* __restrict__ out, int64_t total, int inter, int act) {
     const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
     if (i >= total) return;
     const float g = to_float(x[2 * i]);
     const float u = to_float(x[2 * i + 1]);
-    out[i] = from_float<T>((g / (1.0f + expf(-g))) * u);
+    out[i] = from_float<T>(gate_act(g, act) * u);
 }
 
 // four outputs per thread: 8 inputs in 16 (bfloat16) or 32 (float32) bytes
 template <typename T>
-__global__ void swiglu_vec_kernel(const T* __restrict__ x, T* __restrict__ out, int64_t quads) {
+__global__ void swiglu_vec_kernel(const T* __restrict__ x, T* __restrict__ out, int64_t quads, int act) {
     const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
     if (i >= quads) return;
     const float4 a = Pack4<T>::load(x + 8 * i), b = Pack4<T>::load(x + 8 * i + 4);
-    Pack4<T>::store(out + 4 * i, float4{(a.x / (1.0f + expf(-a.x))) * a.y, (a.z / (1.0f + expf(-a.z))) * a.w,
-                                        (b.x / (1.0f + expf(-b.x))) * b.y, (b.z / (1.0f + expf(-b.z))) * b.w});
+    Pack4<T>::store(out + 4 * i, float4{gate_act(a.x, act) * a.y, gate_act(a.z, act) * a.w,
+                                        gate_act(b.x, act) * b.y, gate_act(b.z, act) * b.w});
 }
 
 template <typename T>
@@ -493,8 +493,9 @@ extern "C" int fsie_rmsnorm(float* residual, const void* delta, const float* wei
     return 0;
 }
 
-extern "C" int fsie_swiglu(const void* x, void* out, int n_tokens, int inter, int dtype, hipStream_t stream) {
+extern "C" int fsie_gated_act(const void* x, void* out, int n_tokens, int inter, int dtype, int act, hipStream_t stream) {
     FSIE_REQUIRE(n_tokens >= 0 && inter > 0, "swiglu: bad sizes T=%d I=%d", n_tokens, inter);
+    FSIE_REQUIRE(act == FSIE_ACT_SILU || act == FSIE_ACT_GELU_TANH, "gated_act: unknown activation %d", act);
     FSIE_REQUIRE(dtype == FSIE_F32 || dtype == FSIE_BF16, "swiglu: unknown dtype %d", dtype);
     const int64_t total = static_cast<int64_t>(n_tokens) * inter;
     if (total == 0) return 0;
@@ -502,14 +503,18 @@ extern "C" int fsie_swiglu(const void* x, void* out, int n_tokens, int inter, in
     const int64_t work = vec ? total / 4 : total;
     const unsigned grid = static_cast<unsigned>(ceil_div64(work, kThreads));
     if (dtype == FSIE_F32) {
-        if (vec) swiglu_vec_kernel<float><<<grid, kThreads, 0, stream>>>(static_cast<const float*>(x), static_cast<float*>(out), work);
-        else swiglu_kernel<float><<<grid, kThreads, 0, stream>>>(static_cast<const float*>(x), static_cast<float*>(out), total, inter);
+        if (vec) swiglu_vec_kernel<float><<<grid, kThreads, 0, stream>>>(static_cast<const float*>(x), static_cast<float*>(out), work, act);
+        else swiglu_kernel<float><<<grid, kThreads, 0, stream>>>(static_cast<const float*>(x), static_cast<float*>(out), total, inter, act);
     } else {
-        if (vec) swiglu_vec_kernel<bf16_t><<<grid, kThreads, 0, stream>>>(static_cast<const bf16_t*>(x), static_cast<bf16_t*>(out), work);
-        else swiglu_kernel<bf16_t><<<grid, kThreads, 0, stream>>>(static_cast<const bf16_t*>(x), static_cast<bf16_t*>(out), total, inter);
+        if (vec) swiglu_vec_kernel<bf16_t><<<grid, kThreads, 0, stream>>>(static_cast<const bf16_t*>(x), static_cast<bf16_t*>(out), work, act);
+        else swiglu_kernel<bf16_t><<<grid, kThreads, 0, stream>>>(static_cast<const bf16_t*>(x), static_cast<bf16_t*>(out), total, inter, act);
     }
     FSIE_CHECK_LAUNCH("swiglu");
     return 0;
+}
+
+extern "C" int fsie_swiglu(const void* x, void* out, int n_tokens, int inter, int dtype, hipStream_t stream) {
+    return fsie_gated_act(x, out, n_tokens, inter, dtype, FSIE_ACT_SILU, stream);
 }
 
 extern "C" int fsie_residual_add(float* residual, const void* delta, int64_t total, int dtype, hipStream_t stream) {

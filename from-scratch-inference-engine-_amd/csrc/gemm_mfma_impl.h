@@ -72,7 +72,7 @@ __device__ __forceinline__ void rotation(double pos, double inv_freq, float* c, 
 template <int MT, int NB, int WAVES, typename OutT, int EPI>
 __global__ __launch_bounds__(WAVES * FSIE_WAVE) void gemm_mfma_skinny_kernel(
     const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, const float* __restrict__ bias,
-    OutT* __restrict__ y, int M, int N, int K, int k_slice, RopeArgs rope) {
+    OutT* __restrict__ y, int M, int N, int K, int k_slice, RopeArgs rope, int act) {
     constexpr bool SWIGLU = EPI == EPI_SWIGLU;
     __shared__ float red[WAVES > 1 ? (WAVES - 1) * NB * MT * FSIE_WAVE * 4 : 1];
     const int lane = threadIdx.x & (FSIE_WAVE - 1);
@@ -282,7 +282,7 @@ __global__ __launch_bounds__(WAVES * FSIE_WAVE) void gemm_mfma_skinny_kernel(
                     const int nn = n0 + nb * 16 + kg * 4 + r;  // even: a gate row, nn + 1 its up row
                     if (nn + 1 < N) {
                         const float g = acc[nb][t][r], u = acc[nb][t][r + 1];
-                        y[static_cast<int64_t>(m) * (N / 2) + nn / 2] = from_float<OutT>((g / (1.0f + expf(-g))) * u);
+                        y[static_cast<int64_t>(m) * (N / 2) + nn / 2] = from_float<OutT>(gate_act(g, act) * u);
                     }
                 }
                 continue;
@@ -307,6 +307,7 @@ struct Call {
     int splits;  // slices of K, each a workgroup row of its own (partial sums out) when > 1
     hipStream_t stream;
     RopeArgs rope;
+    int act = 0;  // EPI_SWIGLU: the gate's activation (FsieGateAct)
 };
 
 template <int MT, int NB, int WAVES, typename OutT, int EPI>
@@ -317,7 +318,7 @@ int launch(const Call& c) {
     const dim3 grid(groups, static_cast<unsigned>(c.splits > 1 ? c.splits : 1));
     gemm_mfma_skinny_kernel<MT, NB, WAVES, OutT, EPI><<<grid, WAVES * FSIE_WAVE, 0, c.stream>>>(
         static_cast<const bf16_t*>(c.x), static_cast<const bf16_t*>(c.w), c.bias, static_cast<OutT*>(c.y), c.M, c.N,
-        c.K, k_slice, c.rope);
+        c.K, k_slice, c.rope, c.act);
     FSIE_CHECK_LAUNCH("gemm_mfma_skinny");
     return 0;
 }

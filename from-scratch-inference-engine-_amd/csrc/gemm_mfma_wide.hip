@@ -64,7 +64,7 @@ template <int MT, int WAVES, int STEPS, int NB, bool SWIGLU, bool FRAGS>
 __global__ __launch_bounds__(WAVES * 64) void gemm_mfma_wide_kernel(const bf16_t* __restrict__ x,
                                                                    const bf16_t* __restrict__ w,
                                                                    float* __restrict__ y, int M, int N, int K,
-                                                                   int k_slice) {
+                                                                   int k_slice, int act) {
     constexpr int KS = 32 * STEPS;
     constexpr int ROWS = 16 * MT;             // rows of X in LDS (rows past M repeat the last one)
     constexpr int UNITS = ROWS * 4 * STEPS;   // 16-byte units of a stage of X
@@ -194,7 +194,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_mfma_wide_kernel(const bf16_t
                 if (m >= M || nn >= N) continue;      // N is a multiple of 4 here (checked by the host)
                 const float g0 = acc[nb][t][0], u0 = acc[nb][t][1], g1 = acc[nb][t][2], u1 = acc[nb][t][3];
                 out[(static_cast<int64_t>(m) * (N / 2) + nn / 2) / 2] =
-                    pack2_bf16((g0 / (1.0f + expf(-g0))) * u0, (g1 / (1.0f + expf(-g1))) * u1);
+                    pack2_bf16(gate_act(g0, act) * u0, gate_act(g1, act) * u1);
             }
         return;
     }
@@ -215,7 +215,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_mfma_wide_kernel(const bf16_t
 
 template <int MT, int WAVES, int STEPS, int NB, bool SWIGLU, bool FRAGS>
 int launch(const bf16_t* x, const bf16_t* w, float* y, int M, int N, int K, int splits, int k_slice,
-           hipStream_t stream) {
+           int act, hipStream_t stream) {
     const int rows = 16 * NB * WAVES;
     const dim3 grid(static_cast<unsigned>((N + rows - 1) / rows), static_cast<unsigned>(splits));
     constexpr int lds = wide_lds_bytes(MT, STEPS);
@@ -229,28 +229,28 @@ int launch(const bf16_t* x, const bf16_t* w, float* y, int M, int N, int K, int 
             return 1;
         }
     }
-    gemm_mfma_wide_kernel<MT, WAVES, STEPS, NB, SWIGLU, FRAGS><<<grid, WAVES * 64, dynamic, stream>>>(x, w, y, M, N, K, k_slice);
+    gemm_mfma_wide_kernel<MT, WAVES, STEPS, NB, SWIGLU, FRAGS><<<grid, WAVES * 64, dynamic, stream>>>(x, w, y, M, N, K, k_slice, act);
     FSIE_CHECK_LAUNCH("gemm_mfma_wide");
     return 0;
 }
 
 template <int WAVES, int STEPS, int NB, bool SWIGLU, bool FRAGS>
-int launch_mt(int mt, const bf16_t* x, const bf16_t* w, float* y, int M, int N, int K, int splits, int k_slice,
+int launch_mt(int mt, const bf16_t* x, const bf16_t* w, float* y, int M, int N, int K, int splits, int k_slice, int act,
               hipStream_t stream) {
     switch (mt) {
-        case 1: return launch<1, WAVES, STEPS, NB, SWIGLU, FRAGS>(x, w, y, M, N, K, splits, k_slice, stream);
-        case 2: return launch<2, WAVES, STEPS, NB, SWIGLU, FRAGS>(x, w, y, M, N, K, splits, k_slice, stream);
+        case 1: return launch<1, WAVES, STEPS, NB, SWIGLU, FRAGS>(x, w, y, M, N, K, splits, k_slice, act, stream);
+        case 2: return launch<2, WAVES, STEPS, NB, SWIGLU, FRAGS>(x, w, y, M, N, K, splits, k_slice, act, stream);
 #if FSIE_WIDE_STEPS <= 4
-        case 3: return launch<3, WAVES, STEPS, NB, SWIGLU, FRAGS>(x, w, y, M, N, K, splits, k_slice, stream);
-        case 4: return launch<4, WAVES, STEPS, NB, SWIGLU, FRAGS>(x, w, y, M, N, K, splits, k_slice, stream);
+        case 3: return launch<3, WAVES, STEPS, NB, SWIGLU, FRAGS>(x, w, y, M, N, K, splits, k_slice, act, stream);
+        case 4: return launch<4, WAVES, STEPS, NB, SWIGLU, FRAGS>(x, w, y, M, N, K, splits, k_slice, act, stream);
         default:
             // five to eight tiles of X (65 to 128 rows): on a fragment-ordered weight, two row blocks a
             // wave, four waves and more
             if constexpr (FRAGS && NB == 2 && WAVES >= 4) {
-                if (mt == 8) return launch<8, WAVES, STEPS, NB, SWIGLU, FRAGS>(x, w, y, M, N, K, splits, k_slice, stream);
-                if (mt == 5) return launch<5, WAVES, STEPS, NB, SWIGLU, FRAGS>(x, w, y, M, N, K, splits, k_slice, stream);
-                if (mt == 6) return launch<6, WAVES, STEPS, NB, SWIGLU, FRAGS>(x, w, y, M, N, K, splits, k_slice, stream);
-                if (mt == 7) return launch<7, WAVES, STEPS, NB, SWIGLU, FRAGS>(x, w, y, M, N, K, splits, k_slice, stream);
+                if (mt == 8) return launch<8, WAVES, STEPS, NB, SWIGLU, FRAGS>(x, w, y, M, N, K, splits, k_slice, act, stream);
+                if (mt == 5) return launch<5, WAVES, STEPS, NB, SWIGLU, FRAGS>(x, w, y, M, N, K, splits, k_slice, act, stream);
+                if (mt == 6) return launch<6, WAVES, STEPS, NB, SWIGLU, FRAGS>(x, w, y, M, N, K, splits, k_slice, act, stream);
+                if (mt == 7) return launch<7, WAVES, STEPS, NB, SWIGLU, FRAGS>(x, w, y, M, N, K, splits, k_slice, act, stream);
             }
             fsie_set_error("gemm_mfma_wide: %d rows only on a fragment-ordered weight with two row blocks a wave and "
                            "at least four waves (N = %d in %d slices gives %d blocks, %d waves)", M, N, splits, NB, WAVES);
@@ -263,21 +263,21 @@ int launch_mt(int mt, const bf16_t* x, const bf16_t* w, float* y, int M, int N, 
 
 template <bool SWIGLU, bool FRAGS>
 int launch_shape_of(int mt, int waves, int blocks, const bf16_t* x, const bf16_t* w, float* y, int M, int N, int K,
-                    int splits, int k_slice, hipStream_t stream) {
+                    int splits, int k_slice, int act, hipStream_t stream) {
     if constexpr (SWIGLU && FRAGS) {  // gate/up of 17 rows and more: any number of waves that deals the rows evenly
-        if (blocks == 2 && waves == 3) return launch_mt<3, FSIE_WIDE_STEPS, 2, true, true>(mt, x, w, y, M, N, K, splits, k_slice, stream);
-        if (blocks == 2 && waves == 5) return launch_mt<5, FSIE_WIDE_STEPS, 2, true, true>(mt, x, w, y, M, N, K, splits, k_slice, stream);
-        if (blocks == 2 && waves == 6) return launch_mt<6, FSIE_WIDE_STEPS, 2, true, true>(mt, x, w, y, M, N, K, splits, k_slice, stream);
-        if (blocks == 2 && waves == 7) return launch_mt<7, FSIE_WIDE_STEPS, 2, true, true>(mt, x, w, y, M, N, K, splits, k_slice, stream);
+        if (blocks == 2 && waves == 3) return launch_mt<3, FSIE_WIDE_STEPS, 2, true, true>(mt, x, w, y, M, N, K, splits, k_slice, act, stream);
+        if (blocks == 2 && waves == 5) return launch_mt<5, FSIE_WIDE_STEPS, 2, true, true>(mt, x, w, y, M, N, K, splits, k_slice, act, stream);
+        if (blocks == 2 && waves == 6) return launch_mt<6, FSIE_WIDE_STEPS, 2, true, true>(mt, x, w, y, M, N, K, splits, k_slice, act, stream);
+        if (blocks == 2 && waves == 7) return launch_mt<7, FSIE_WIDE_STEPS, 2, true, true>(mt, x, w, y, M, N, K, splits, k_slice, act, stream);
     }
     if (blocks == 2) {
-        if (waves == 8) return launch_mt<8, FSIE_WIDE_STEPS, 2, SWIGLU, FRAGS>(mt, x, w, y, M, N, K, splits, k_slice, stream);
-        if (waves == 2) return launch_mt<2, FSIE_WIDE_STEPS, 2, SWIGLU, FRAGS>(mt, x, w, y, M, N, K, splits, k_slice, stream);
-        return launch_mt<4, FSIE_WIDE_STEPS, 2, SWIGLU, FRAGS>(mt, x, w, y, M, N, K, splits, k_slice, stream);
+        if (waves == 8) return launch_mt<8, FSIE_WIDE_STEPS, 2, SWIGLU, FRAGS>(mt, x, w, y, M, N, K, splits, k_slice, act, stream);
+        if (waves == 2) return launch_mt<2, FSIE_WIDE_STEPS, 2, SWIGLU, FRAGS>(mt, x, w, y, M, N, K, splits, k_slice, act, stream);
+        return launch_mt<4, FSIE_WIDE_STEPS, 2, SWIGLU, FRAGS>(mt, x, w, y, M, N, K, splits, k_slice, act, stream);
     }
-    if (waves == 8) return launch_mt<8, FSIE_WIDE_STEPS, 1, SWIGLU, FRAGS>(mt, x, w, y, M, N, K, splits, k_slice, stream);
-    if (waves == 2) return launch_mt<2, FSIE_WIDE_STEPS, 1, SWIGLU, FRAGS>(mt, x, w, y, M, N, K, splits, k_slice, stream);
-    return launch_mt<4, FSIE_WIDE_STEPS, 1, SWIGLU, FRAGS>(mt, x, w, y, M, N, K, splits, k_slice, stream);
+    if (waves == 8) return launch_mt<8, FSIE_WIDE_STEPS, 1, SWIGLU, FRAGS>(mt, x, w, y, M, N, K, splits, k_slice, act, stream);
+    if (waves == 2) return launch_mt<2, FSIE_WIDE_STEPS, 1, SWIGLU, FRAGS>(mt, x, w, y, M, N, K, splits, k_slice, act, stream);
+    return launch_mt<4, FSIE_WIDE_STEPS, 1, SWIGLU, FRAGS>(mt, x, w, y, M, N, K, splits, k_slice, act, stream);
 }
 
 // One thread a 16-byte unit of the copy: unit ((block, step), lane) holds the 8 values at row
@@ -443,14 +443,16 @@ extern "C" int fsie_gemm_mfma_wide(const void* x, const void* w, float* y, int M
     launch_shape(mt, N, splits, waves, blocks, false, frags != 0);
     const bf16_t* xp = static_cast<const bf16_t*>(x);
     const bf16_t* wq = static_cast<const bf16_t*>(w);
-    if (frags) return launch_shape_of<false, true>(mt, waves, blocks, xp, wq, y, M, N, K, splits, k_slice, stream);
-    return launch_shape_of<false, false>(mt, waves, blocks, xp, wq, y, M, N, K, splits, k_slice, stream);
+    if (frags) return launch_shape_of<false, true>(mt, waves, blocks, xp, wq, y, M, N, K, splits, k_slice, 0, stream);
+    return launch_shape_of<false, false>(mt, waves, blocks, xp, wq, y, M, N, K, splits, k_slice, 0, stream);
 }
 
 // The same product with the rows of w as gate and up in turn: y is bfloat16 [M, N / 2], silu(gate) * up.
 // N a multiple of 4; one slice of K.
-extern "C" int fsie_gemm_mfma_wide_swiglu(const void* x, const void* w, void* y, int M, int N, int K, int waves,
-                                          int blocks, int frags, hipStream_t stream) {
+// act: the gate's activation (FsieGateAct: 0 SiLU, 1 GELU in its tanh form).
+extern "C" int fsie_gemm_mfma_wide_gated(const void* x, const void* w, void* y, int M, int N, int K, int waves,
+                                         int blocks, int frags, int act, hipStream_t stream) {
+    FSIE_REQUIRE(act == FSIE_ACT_SILU || act == FSIE_ACT_GELU_TANH, "gemm_mfma_wide_gated: unknown activation %d", act);
     FSIE_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm_mfma_wide_swiglu: bad sizes M=%d N=%d K=%d", M, N, K);
     FSIE_REQUIRE(M <= (frags ? FSIE_GEMM_MFMA_WIDE_MAX_M : FSIE_GEMM_MFMA_SKINNY_MAX_M),
                  "gemm_mfma_wide_swiglu: at most %d rows (%d on a fragment-ordered weight), got %d",
@@ -470,8 +472,13 @@ extern "C" int fsie_gemm_mfma_wide_swiglu(const void* x, const void* w, void* y,
     const bf16_t* xp = static_cast<const bf16_t*>(x);
     const bf16_t* wq = static_cast<const bf16_t*>(w);
     float* yp = static_cast<float*>(y);
-    if (frags) return launch_shape_of<true, true>(mt, waves, blocks, xp, wq, yp, M, N, K, 1, k_slice, stream);
-    return launch_shape_of<true, false>(mt, waves, blocks, xp, wq, yp, M, N, K, 1, k_slice, stream);
+    if (frags) return launch_shape_of<true, true>(mt, waves, blocks, xp, wq, yp, M, N, K, 1, k_slice, act, stream);
+    return launch_shape_of<true, false>(mt, waves, blocks, xp, wq, yp, M, N, K, 1, k_slice, act, stream);
+}
+
+extern "C" int fsie_gemm_mfma_wide_swiglu(const void* x, const void* w, void* y, int M, int N, int K, int waves,
+                                          int blocks, int frags, hipStream_t stream) {
+    return fsie_gemm_mfma_wide_gated(x, w, y, M, N, K, waves, blocks, frags, FSIE_ACT_SILU, stream);
 }
 
 // The copy of a bfloat16 matrix w [N, K] in the order of the matrix instruction's A fragments, for

@@ -1,0 +1,144 @@
+// Norms and activations beyond the plain pre-norm layer: the norm of a sublayer's output fused with
+// the residual sum and the next norm (a layer with a norm before and after every sublayer), the norm
+// of every head of a mixer's output fused with its gate, and the soft cap of the logits.
+// All arithmetic is float32; T is the type of activations (float or bfloat16).
+#include "common.h"
+#include "api.h"
+
+namespace {
+
+constexpr int kThreads = 256;
+
+// One block per output row r; source row = rows ? rows[r] : r.
+//   y = delta[row]                          (one array of T, or the sum in order of n_parts float32 arrays)
+//   d = y * rsqrt(mean(y^2) + post_eps) * post_weight
+//   v = residual[row] + d;                  if write_back: residual[row] = v
+//   out[r] = v * rsqrt(mean(v^2) + eps) * weight
+// The row is kept in LDS between the passes (hidden floats).
+template <typename T>
+__global__ __launch_bounds__(kThreads) void sandwich_norm_kernel(
+    float* __restrict__ residual, const T* __restrict__ delta, const float* __restrict__ post_weight, float post_eps,
+    const float* __restrict__ weight, float eps, T* __restrict__ out, const int32_t* __restrict__ rows, int hidden,
+    int write_back, int n_parts, int64_t part_stride) {
+    extern __shared__ float row_buf[];
+    __shared__ float scratch[16];
+    const int r = blockIdx.x;
+    const int64_t row = rows ? rows[r] : r;
+    float* res = residual + row * hidden;
+    const T* del = n_parts ? nullptr : delta + row * hidden;
+    const float* parts = n_parts ? reinterpret_cast<const float*>(delta) + row * hidden : nullptr;
+    float sum_sq = 0.f;
+    for (int j = threadIdx.x; j < hidden; j += kThreads) {
+        float y;
+        if (del) {
+            y = to_float(del[j]);
+        } else {
+            y = 0.f;
+            for (int s = 0; s < n_parts; ++s) y += parts[s * part_stride + j];
+        }
+        row_buf[j] = y;
+        sum_sq += y * y;
+    }
+    const float post_scale = 1.0f / sqrtf(block_sum(sum_sq, scratch) / static_cast<float>(hidden) + post_eps);
+    sum_sq = 0.f;
+    for (int j = threadIdx.x; j < hidden; j += kThreads) {
+        const float v = res[j] + (row_buf[j] * post_scale) * post_weight[j];
+        row_buf[j] = v;
+        if (write_back) res[j] = v;
+        sum_sq += v * v;
+    }
+    const float scale = 1.0f / sqrtf(block_sum(sum_sq, scratch) / static_cast<float>(hidden) + eps);
+    T* dst = out + static_cast<int64_t>(r) * hidden;
+    for (int j = threadIdx.x; j < hidden; j += kThreads) dst[j] = from_float<T>((row_buf[j] * scale) * weight[j]);
+}
+
+// One wave per (token, head): o [tokens][heads * width] float32 is normalised over the `width` values of
+// the head (plain weight [width], shared by the heads) and multiplied by act(gate) of the same place;
+// gate [tokens][gate_stride] of T (the columns of the head start at h * width).
+template <typename T>
+__global__ __launch_bounds__(kThreads) void gated_headnorm_kernel(const float* __restrict__ o, const T* __restrict__ gate,
+                                                                  int64_t gate_stride, const float* __restrict__ weight,
+                                                                  T* __restrict__ out, int64_t n_runs, int heads, int width,
+                                                                  float eps, int act) {
+    const int lane = threadIdx.x & (FSIE_WAVE - 1);
+    const int64_t run = static_cast<int64_t>(blockIdx.x) * (kThreads / FSIE_WAVE) + threadIdx.x / FSIE_WAVE;
+    if (run >= n_runs) return;
+    const int64_t t = run / heads;
+    const int h = static_cast<int>(run - t * heads);
+    const float* src = o + (t * heads + h) * width;
+    const T* g = gate + t * gate_stride + static_cast<int64_t>(h) * width;
+    T* dst = out + (t * heads + h) * width;
+    float sum = 0.f;
+    for (int i = lane; i < width; i += FSIE_WAVE) sum += src[i] * src[i];
+    sum = wave_sum(sum);
+    const float scale = 1.0f / sqrtf(sum / static_cast<float>(width) + eps);
+    for (int i = lane; i < width; i += FSIE_WAVE)
+        dst[i] = from_float<T>(((src[i] * scale) * weight[i]) * gate_act(to_float(g[i]), act));
+}
+
+__global__ void softcap_kernel(float* __restrict__ x, int64_t n, float cap, float inv_cap) {
+    const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i < n) x[i] = cap * tanhf(x[i] * inv_cap);
+}
+
+}  // namespace
+
+// The norm of a sublayer's output, the residual sum and the next norm in one pass (see the kernel).
+// delta: [total_rows][hidden] of the activations' type, or with n_parts > 0 that many float32 arrays
+// [total_rows][hidden] one after the other.  rows (or null): the n_rows source rows to work on.
+extern "C" int fsie_sandwich_norm(float* residual, const void* delta, const float* post_weight, float post_eps,
+                                  const float* weight, float eps, void* out, const int32_t* rows, int n_rows, int hidden,
+                                  int dtype, int write_back, int n_parts, int total_rows, hipStream_t stream) {
+    FSIE_REQUIRE(n_rows >= 0 && hidden > 0 && hidden <= 16384, "sandwich_norm: bad sizes rows=%d hidden=%d (at most 16384)",
+                 n_rows, hidden);
+    FSIE_REQUIRE(dtype == FSIE_F32 || dtype == FSIE_BF16, "sandwich_norm: unknown dtype %d", dtype);
+    FSIE_REQUIRE(residual && delta && post_weight && weight && out, "sandwich_norm: missing operand");
+    FSIE_REQUIRE(n_parts >= 0 && n_parts <= FSIE_GEMM_MAX_SPLITS, "sandwich_norm: 0 to %d partial sums, got %d",
+                 FSIE_GEMM_MAX_SPLITS, n_parts);
+    FSIE_REQUIRE(!(write_back && rows), "sandwich_norm: chosen rows are read, not written back");
+    if (n_rows == 0) return 0;
+    const int64_t part_stride = static_cast<int64_t>(total_rows) * hidden;
+    const size_t lds = sizeof(float) * hidden;
+    if (dtype == FSIE_F32) {
+        sandwich_norm_kernel<float><<<n_rows, kThreads, lds, stream>>>(residual, static_cast<const float*>(delta), post_weight,
+                                                                     post_eps, weight, eps, static_cast<float*>(out), rows,
+                                                                     hidden, write_back, n_parts, part_stride);
+    } else {
+        sandwich_norm_kernel<bf16_t><<<n_rows, kThreads, lds, stream>>>(residual, static_cast<const bf16_t*>(delta), post_weight,
+                                                                      post_eps, weight, eps, static_cast<bf16_t*>(out), rows,
+                                                                      hidden, write_back, n_parts, part_stride);
+    }
+    FSIE_CHECK_LAUNCH("sandwich_norm");
+    return 0;
+}
+
+extern "C" int fsie_gated_headnorm(const float* o, const void* gate, int64_t gate_stride, const float* weight, void* out,
+                                   int n_tokens, int heads, int width, float eps, int act, int dtype, hipStream_t stream) {
+    FSIE_REQUIRE(n_tokens >= 0 && heads > 0 && width > 0, "gated_headnorm: bad sizes T=%d heads=%d width=%d", n_tokens, heads,
+                 width);
+    FSIE_REQUIRE(dtype == FSIE_F32 || dtype == FSIE_BF16, "gated_headnorm: unknown dtype %d", dtype);
+    FSIE_REQUIRE(act == FSIE_ACT_SILU || act == FSIE_ACT_GELU_TANH, "gated_headnorm: unknown activation %d", act);
+    FSIE_REQUIRE(o && gate && weight && out && gate_stride >= static_cast<int64_t>(heads) * width,
+                 "gated_headnorm: missing operand or a gate row shorter than the heads");
+    if (n_tokens == 0) return 0;
+    const int64_t runs = static_cast<int64_t>(n_tokens) * heads;
+    const unsigned grid = static_cast<unsigned>(ceil_div64(runs, kThreads / FSIE_WAVE));
+    if (dtype == FSIE_F32) {
+        gated_headnorm_kernel<float><<<grid, kThreads, 0, stream>>>(o, static_cast<const float*>(gate), gate_stride, weight,
+                                                                  static_cast<float*>(out), runs, heads, width, eps, act);
+    } else {
+        gated_headnorm_kernel<bf16_t><<<grid, kThreads, 0, stream>>>(o, static_cast<const bf16_t*>(gate), gate_stride, weight,
+                                                                   static_cast<bf16_t*>(out), runs, heads, width, eps, act);
+    }
+    FSIE_CHECK_LAUNCH("gated_headnorm");
+    return 0;
+}
+
+// x <- cap * tanh(x / cap), in place, float32.
+extern "C" int fsie_softcap(float* x, int64_t n, float cap, hipStream_t stream) {
+    FSIE_REQUIRE(n >= 0 && cap > 0.f, "softcap: bad arguments n=%lld cap=%f", static_cast<long long>(n), cap);
+    if (n == 0) return 0;
+    softcap_kernel<<<static_cast<unsigned>(ceil_div64(n, kThreads)), kThreads, 0, stream>>>(x, n, cap, 1.0f / cap);
+    FSIE_CHECK_LAUNCH("softcap");
+    return 0;
+}

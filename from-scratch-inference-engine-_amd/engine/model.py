@@ -22,7 +22,7 @@ from ..config.base import ModelConfig, read_config_json
 from ..models.registry import build_model_spec, parse_config
 from ..models.spec import ModelSpec
 from ..parts.base import HiddenState, prepare_parts
-from ..weights.loader import fill_parts, load_weights
+from ..weights.loader import fill_parts, load_weights, tensor_shapes
 from ..weights.random_init import random_tensor, expected_tensors
 from .context import PinnedStaging, StepContext, StepEntry, build_context, filler_entry
 
@@ -104,7 +104,7 @@ class Model:
         """``weight_copies=False``: no second, fragment-ordered copy of the large matrices (half
         the memory; decode steps then read rows and are some 8 % slower)."""
         device = _require_gpu(device)
-        config = parse_config(read_config_json(model_dir))
+        config = parse_config(read_config_json(model_dir)).completed_from(tensor_shapes(Path(model_dir)))
         model = cls(build_model_spec(config), dtype, device)
         model.weight_bytes = load_weights(Path(model_dir), model.spec.bindings, model.dtype, device,
                                           model.spec.ignore_unexpected)

@@ -22,7 +22,7 @@ import sys
 from pathlib import Path
 
 PAGE_SIZE = 16
-MAX_LIVE_REQUESTS = 16
+MAX_LIVE_REQUESTS = 4
 
 
 def main(argv=None) -> int:
@@ -33,6 +33,8 @@ def main(argv=None) -> int:
     parser.add_argument("--max-tokens", type=int, required=True,
                         help="most tokens live requests hold at any time (each rounded up to 64)")
     parser.add_argument("--page-size", type=int, default=PAGE_SIZE)
+    parser.add_argument("--max-requests", type=int, default=MAX_LIVE_REQUESTS,
+                        help="state slots: the most requests that are live at any time")
     args = parser.parse_args(argv)
 
     print("[trace_run] loading the kernel library and the model", file=sys.stderr, flush=True)
@@ -47,7 +49,7 @@ def main(argv=None) -> int:
     model = Model.from_pretrained(args.model, dtype=args.dtype, device="cuda:0")
     page = max(1, args.page_size)
     num_pages = -(-max(args.max_tokens, 64) // page)
-    runner = Runner(model, page_size=page, num_pages=num_pages, max_requests=MAX_LIVE_REQUESTS)
+    runner = Runner(model, page_size=page, num_pages=num_pages, max_requests=max(1, args.max_requests))
     out_dir = Path(args.out)
     out_dir.mkdir(parents=True, exist_ok=True)
     print(f"[trace_run] ready: {args.dtype}, {num_pages} pages of {page} tokens", file=sys.stderr, flush=True)

@@ -31,12 +31,14 @@ def known_architectures():
 
 
 def _ensure_builtin() -> None:
-    from . import qwen2  # noqa: F401  (registers itself)
+    from . import gilozen, qwen2  # noqa: F401  (they register themselves)
 
 
 def architecture_of(raw: Mapping) -> Architecture:
     _ensure_builtin()
     archs = raw.get("architectures")
+    if isinstance(raw.get("architecture"), str) and not archs:
+        archs = [raw["architecture"]]  # (some configurations name their one architecture under this key)
     if not archs or not isinstance(archs, list):
         raise ConfigError("config.json: 'architectures' is missing; known architectures: "
                           + ", ".join(sorted(_ARCHITECTURES)))
@@ -52,7 +54,9 @@ def parse_config(raw: Mapping) -> ModelConfig:
 
 
 def load_config(model_dir) -> ModelConfig:
-    return parse_config(read_config_json(model_dir))
+    from ..weights.loader import tensor_shapes
+
+    return parse_config(read_config_json(model_dir)).completed_from(tensor_shapes(model_dir))
 
 
 def build_model_spec(config: ModelConfig) -> ModelSpec:

@@ -11,7 +11,8 @@ from .functions import (FragmentOrdered, attention_merge, attention_mfma, attent
                         gemm_mfma_skinny_rope, gemm_mfma_wide, gemm_mfma_wide_best_splits, gemm_mfma_wide_splits_ok,
                         gemm_mfma_wide_swiglu, gemm_mfma_wide_takes, random_fill,
                         residual_add,
-                        rmsnorm, rmsnorm_plain, rope_kv_write, rope_table, sample, swiglu, zero_pages, zero_rows)
+                        rmsnorm, rmsnorm_plain, rope_kv_write, rope_table, sample, swiglu, zero_pages, zero_rows,
+                        gate_act_code, gated_headnorm, gla_scan, head_gemm, latent_prep, rope_pairs, sandwich_norm, softcap)
 from .library import KernelError, KernelLibraryMissing, load
 from .tuning import disable_library_tuning, enable_library_tuning, library_mm, library_tuning_enabled
 
@@ -20,4 +21,5 @@ __all__ = ["FragmentOrdered", "KernelError", "KernelLibraryMissing", "attention_
            "attention_tile_tokens", "bias_add", "compute_units", "disable_library_tuning", "dtype_code", "embedding",
            "enable_library_tuning", "fragment_order", "gemm", "gemm_mfma_fp32", "gemm_mfma_skinny", "gemm_mfma_skinny_rope", "gemm_mfma_wide",
            "gemm_mfma_wide_best_splits", "gemm_mfma_wide_splits_ok", "gemm_mfma_wide_swiglu", "gemm_mfma_wide_takes", "library_mm", "library_tuning_enabled", "load", "random_fill", "residual_add",
-           "rmsnorm", "rmsnorm_plain", "rope_kv_write", "rope_table", "sample", "swiglu", "zero_pages", "zero_rows"]
+           "rmsnorm", "rmsnorm_plain", "rope_kv_write", "rope_table", "sample", "swiglu", "zero_pages", "zero_rows",
+           "gate_act_code", "gated_headnorm", "gla_scan", "head_gemm", "latent_prep", "rope_pairs", "sandwich_norm", "softcap"]

@@ -159,8 +159,18 @@ def random_fill(out: torch.Tensor, key: int, init: str, std: float = 0.0) -> tor
     return out
 
 
-def swiglu(x: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """silu(x[:, 0::2]) * x[:, 1::2] for x [T, 2I] (gate and up interleaved)."""
+GATE_ACTS = {"silu": 0, "gelu_tanh": 1}  # the activations of a gate that the kernels know
+
+
+def gate_act_code(act: str) -> int:
+    try:
+        return GATE_ACTS[act]
+    except KeyError:
+        raise KernelError(f"unknown gate activation '{act}' (known: {sorted(GATE_ACTS)})") from None
+
+
+def swiglu(x: torch.Tensor, out: Optional[torch.Tensor] = None, act: str = "silu") -> torch.Tensor:
+    """act(x[:, 0::2]) * x[:, 1::2] for x [T, 2I] (gate and up interleaved); ``act``: "silu" or "gelu_tanh"."""
     _need(x, "swiglu input", ndim=2)
     t, two_i = x.shape
     if two_i % 2:
@@ -169,7 +179,7 @@ def swiglu(x: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
     if out is None:
         out = torch.empty((t, inter), dtype=x.dtype, device=x.device)
     _need(out, "swiglu out", dtype=x.dtype, shape=(t, inter))
-    check(load().fsie_swiglu(x.data_ptr(), out.data_ptr(), t, inter, dtype_code(x.dtype), _stream()))
+    check(load().fsie_gated_act(x.data_ptr(), out.data_ptr(), t, inter, dtype_code(x.dtype), gate_act_code(act), _stream()))
     return out
 
 
@@ -311,11 +321,12 @@ def gemm_mfma_skinny(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch
     out_dtype = out_dtype or x.dtype
     if out_dtype not in (torch.bfloat16, torch.float32):
         raise KernelError(f"gemm: output {out_dtype} is not offered")
-    if epilogue not in ("plain", "swiglu"):
+    if epilogue not in ("plain", "swiglu", "geglu_tanh"):
         raise KernelError(f"gemm: unknown epilogue '{epilogue}'")
-    if epilogue == "swiglu" and n % 2:
+    gated = epilogue != "plain"  # "geglu_tanh": the same with GELU (tanh form) on the gate
+    if gated and n % 2:
         raise KernelError(f"gemm: the swiglu epilogue needs an even number of weight rows, found {n}")
-    n_out = n // 2 if epilogue == "swiglu" else n
+    n_out = n // 2 if gated else n
     shape = (m, n_out)
     if splits != 1:
         if splits not in GEMM_SPLITS or epilogue != "plain" or bias is not None:
@@ -325,7 +336,8 @@ def gemm_mfma_skinny(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch
         out = torch.empty(shape, dtype=out_dtype, device=x.device)
     _need(out, "gemm out", dtype=out_dtype, shape=shape)
     check(load().fsie_gemm_mfma_skinny(x.data_ptr(), weight.data_ptr(), _ptr(bias), out.data_ptr(), m, n, k,
-                                       int(out_dtype == torch.float32), waves, blocks, int(epilogue == "swiglu"),
+                                       int(out_dtype == torch.float32), waves, blocks,
+                                       {"plain": 0, "swiglu": 1, "geglu_tanh": 2}[epilogue],
                                        splits, _stream()))
     return out
 
@@ -389,7 +401,7 @@ def gemm_mfma_wide_splits_ok(k: int, splits: int) -> bool:
 
 
 def gemm_mfma_wide_swiglu(x: torch.Tensor, weight: torch.Tensor, waves: int = 0, blocks: int = 0,
-                          out: Optional[torch.Tensor] = None) -> torch.Tensor:
+                          out: Optional[torch.Tensor] = None, act: str = "silu") -> torch.Tensor:
     """silu(gate) * up [M, N/2] (bfloat16) of x [M, K] and a weight [N, K] whose rows are gate and up
     in turn (or its ``FragmentOrdered`` copy), by the kernel that shares x through LDS; up to 64
     rows, N a multiple of 4, K of 128."""
@@ -401,8 +413,8 @@ def gemm_mfma_wide_swiglu(x: torch.Tensor, weight: torch.Tensor, waves: int = 0,
     if out is None:
         out = torch.empty((m, n // 2), dtype=torch.bfloat16, device=x.device)
     _need(out, "gemm out", dtype=torch.bfloat16, shape=(m, n // 2))
-    check(load().fsie_gemm_mfma_wide_swiglu(x.data_ptr(), wptr, out.data_ptr(), m, n, k, waves, blocks, frags,
-                                            _stream()))
+    check(load().fsie_gemm_mfma_wide_gated(x.data_ptr(), wptr, out.data_ptr(), m, n, k, waves, blocks, frags,
+                                           gate_act_code(act), _stream()))
     return out
 
 
@@ -499,8 +511,11 @@ def attention_tile_tokens(n_heads: int, n_kv: int) -> int:
 def attention_scalar(q: torch.Tensor, q_stride: int, k_pool: torch.Tensor, v_pool: torch.Tensor,
                      block_tables: torch.Tensor, items: torch.Tensor, n_items: int, out: torch.Tensor,
                      partials: Optional[torch.Tensor], n_heads: int, n_kv: int, head_dim: int,
-                     window: Optional[int], scale: float, n_query_rows: int) -> torch.Tensor:
-    """Attention of the work items over the paged cache (float32 arithmetic).
+                     window: Optional[int], scale: float, n_query_rows: int,
+                     sinks: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Attention of the work items over the paged cache (float32 arithmetic).  ``sinks`` (float32 [n_heads],
+    here and in the other attention functions): exp(sinks[h]) is one more term of the denominator of
+    head h's softmax, with no key and no value.
 
     ``q`` is a view into rows of stride ``q_stride`` elements whose first n_heads*head_dim columns
     are the queries; ``out`` is [n_query_rows, n_heads*head_dim]."""
@@ -523,7 +538,8 @@ def attention_scalar(q: torch.Tensor, q_stride: int, k_pool: torch.Tensor, v_poo
     check(load().fsie_attention_scalar(q.data_ptr(), q_stride, k_pool.data_ptr(), v_pool.data_ptr(),
                                        block_tables.data_ptr(), block_tables.shape[1], items.data_ptr(),
                                        n_items, out.data_ptr(), _ptr(partials), n_heads, n_kv, head_dim,
-                                       page_size, int(window or 0), float(scale), dtype_code(q.dtype), _stream()))
+                                       page_size, int(window or 0), float(scale), dtype_code(q.dtype),
+                                       _sinks_ptr(sinks, n_heads), _stream()))
     return out
 
 
@@ -545,7 +561,8 @@ def attention_mfma_max_waves(head_dim: int) -> int:
 def attention_mfma(q: torch.Tensor, q_stride: int, k_pool: torch.Tensor, v_pool: torch.Tensor,
                    block_tables: torch.Tensor, items: torch.Tensor, n_items: int, out: torch.Tensor,
                    partials: Optional[torch.Tensor], n_heads: int, n_kv: int, head_dim: int,
-                   window: Optional[int], scale: float, n_query_rows: int, large: bool, waves: int = 1) -> torch.Tensor:
+                   window: Optional[int], scale: float, n_query_rows: int, large: bool, waves: int = 1,
+                   sinks: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Attention of the work items over the paged cache on the matrix cores (bfloat16; head_dim a
     multiple of 16; page size a multiple of 4).  ``items`` may be a view into a longer table.
     ``waves`` waves of a workgroup split each item's keys and combine inside the workgroup."""
@@ -568,7 +585,8 @@ def attention_mfma(q: torch.Tensor, q_stride: int, k_pool: torch.Tensor, v_pool:
     check(load().fsie_attention_mfma(q.data_ptr(), q_stride, k_pool.data_ptr(), v_pool.data_ptr(),
                                      block_tables.data_ptr(), block_tables.shape[1], items.data_ptr(), n_items,
                                      out.data_ptr(), _ptr(partials), n_heads, n_kv, head_dim, page_size,
-                                     int(window or 0), float(scale), int(large), int(waves), _stream()))
+                                     int(window or 0), float(scale), int(large), int(waves),
+                                     _sinks_ptr(sinks, n_heads), _stream()))
     return out
 
 
@@ -625,7 +643,7 @@ def attention_mfma_lds_ok(head_dim: int, page_size: int) -> bool:
 def attention_mfma_lds(q: torch.Tensor, q_stride: int, k_pool: torch.Tensor, v_pool: torch.Tensor,
                        block_tables: torch.Tensor, items: torch.Tensor, groups: torch.Tensor, n_groups: int,
                        out: torch.Tensor, n_heads: int, n_kv: int, head_dim: int, window: Optional[int], scale: float,
-                       n_query_rows: int) -> torch.Tensor:
+                       n_query_rows: int, sinks: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Attention of large work items (long portions) with the keys and values of a block staged in
     LDS for four tiles at once.  ``groups`` int32 [n, 2]: index in ``items`` of a group's first
     tile and its number of tiles (1..4, consecutive tiles of one request)."""
@@ -647,19 +665,28 @@ def attention_mfma_lds(q: torch.Tensor, q_stride: int, k_pool: torch.Tensor, v_p
     check(load().fsie_attention_mfma_lds(q.data_ptr(), q_stride, k_pool.data_ptr(), v_pool.data_ptr(),
                                          block_tables.data_ptr(), block_tables.shape[1], items.data_ptr(),
                                          groups.data_ptr(), n_groups, out.data_ptr(), n_heads, n_kv, head_dim,
-                                         page_size, int(window or 0), float(scale), _stream()))
+                                         page_size, int(window or 0), float(scale), _sinks_ptr(sinks, n_heads),
+                                         _stream()))
     return out
 
 
+def _sinks_ptr(sinks: Optional[torch.Tensor], n_heads: int) -> Optional[int]:
+    if sinks is None:
+        return None
+    _need(sinks, "attention sinks", dtype=torch.float32, shape=(n_heads,))
+    return sinks.data_ptr()
+
+
 def attention_merge(partials: torch.Tensor, merges: torch.Tensor, n_merges: int, out: torch.Tensor,
-                    n_heads: int, head_dim: int) -> torch.Tensor:
+                    n_heads: int, head_dim: int, sinks: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``sinks``: added to the denominator once, after the splits (the items that left the records ignored it)."""
     _need(partials, "attention partials", dtype=torch.float32, ndim=1)
     _need(merges, "attention merges", dtype=torch.int32, ndim=2)
     if merges.shape[1] != ATTN_MERGE_INTS or merges.shape[0] < n_merges:
         raise KernelError(f"attention merges: shape {tuple(merges.shape)} does not hold {n_merges} items")
     _need(out, "attention out", ndim=2)
     check(load().fsie_attention_merge(partials.data_ptr(), merges.data_ptr(), n_merges, out.data_ptr(),
-                                      n_heads, head_dim, dtype_code(out.dtype), _stream()))
+                                      n_heads, head_dim, dtype_code(out.dtype), _sinks_ptr(sinks, n_heads), _stream()))
     return out
 
 
@@ -684,4 +711,165 @@ def sample(logits: torch.Tensor, temperature: Optional[torch.Tensor] = None,
     _need(out, "sample out", dtype=torch.int32, shape=(n,))
     check(load().fsie_sample(logits.data_ptr(), n, v, _ptr(temperature), _ptr(top_k), _ptr(top_p),
                              _ptr(uniform), out.data_ptr(), _stream()))
+    return out
+
+
+# ---------------------------------------------------------------------------------------------
+# a layer with a norm before and after every sublayer; norms of heads with a gate; the logits' cap
+# ---------------------------------------------------------------------------------------------
+def sandwich_norm(residual: torch.Tensor, delta: torch.Tensor, post_weight: torch.Tensor, post_eps: float,
+                  weight: torch.Tensor, eps: float, out_dtype: torch.dtype, rows: Optional[torch.Tensor] = None,
+                  write_back: bool = False) -> torch.Tensor:
+    """``v = residual + rmsnorm(delta; post_weight, post_eps)``, then ``rmsnorm(v; weight, eps)`` in
+    ``out_dtype``, one pass.  ``delta`` as for ``rmsnorm``; ``write_back`` stores v into ``residual``
+    (not with ``rows``, which selects the rows to work on)."""
+    _need(residual, "sandwich_norm residual", dtype=torch.float32, ndim=2)
+    t, h = residual.shape
+    _need(weight, "sandwich_norm weight", dtype=torch.float32, shape=(h,))
+    _need(post_weight, "sandwich_norm post weight", dtype=torch.float32, shape=(h,))
+    n_parts = 0
+    if delta.ndim == 3:
+        n_parts = delta.shape[0]
+        _need(delta, "sandwich_norm delta parts", dtype=torch.float32, shape=(n_parts, t, h))
+        if not 1 <= n_parts <= GEMM_MAX_SPLITS:
+            raise KernelError(f"sandwich_norm: {n_parts} partial sums; up to {GEMM_MAX_SPLITS} are taken")
+    else:
+        _need(delta, "sandwich_norm delta", dtype=out_dtype, shape=(t, h))
+    n_rows = t
+    if rows is not None:
+        _need(rows, "sandwich_norm rows", dtype=torch.int32, ndim=1)
+        n_rows = rows.shape[0]
+        if write_back:
+            raise KernelError("sandwich_norm: chosen rows are not written back")
+    out = torch.empty((n_rows, h), dtype=out_dtype, device=residual.device)
+    check(load().fsie_sandwich_norm(residual.data_ptr(), delta.data_ptr(), post_weight.data_ptr(), float(post_eps),
+                                    weight.data_ptr(), float(eps), out.data_ptr(), _ptr(rows), n_rows, h,
+                                    dtype_code(out_dtype), int(write_back), n_parts, t, _stream()))
+    return out
+
+
+def gated_headnorm(o: torch.Tensor, gate: torch.Tensor, weight: torch.Tensor, eps: float, heads: int,
+                   act: str = "silu") -> torch.Tensor:
+    """``rmsnorm(o[t, h]; weight, eps) * act(gate[t, h])`` for every token and head: ``o`` float32
+    [T, heads * width], ``weight`` float32 [width] (shared by the heads), ``gate`` [T, heads * width] in the
+    activations' type (it may be columns of wider rows); the result has the gate's type."""
+    _need(o, "gated_headnorm o", dtype=torch.float32, ndim=2)
+    _need(weight, "gated_headnorm weight", dtype=torch.float32, ndim=1)
+    t, total = o.shape
+    width = weight.shape[0]
+    if total != heads * width:
+        raise KernelError(f"gated_headnorm: rows of {total} values are not {heads} heads of {width}")
+    if not gate.is_cuda or gate.dim() != 2 or gate.stride(1) != 1 or tuple(gate.shape) != (t, total):
+        raise KernelError("gated_headnorm gate: must be [T, heads * width] on the GPU with contiguous rows")
+    out = torch.empty((t, total), dtype=gate.dtype, device=o.device)
+    check(load().fsie_gated_headnorm(o.data_ptr(), gate.data_ptr(), gate.stride(0), weight.data_ptr(), out.data_ptr(), t,
+                                     heads, width, float(eps), gate_act_code(act), dtype_code(gate.dtype), _stream()))
+    return out
+
+
+def softcap(x: torch.Tensor, cap: float) -> torch.Tensor:
+    """``x <- cap * tanh(x / cap)`` in place (float32)."""
+    _need(x, "softcap x", dtype=torch.float32)
+    check(load().fsie_softcap(x.data_ptr(), x.numel(), float(cap), _stream()))
+    return x
+
+
+# ---------------------------------------------------------------------------------------------
+# gated linear attention
+# ---------------------------------------------------------------------------------------------
+def gla_scan(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, z: torch.Tensor, state: torch.Tensor,
+             q_starts: torch.Tensor, seq_slots: torch.Tensor, heads: int, dim: int, vdim: int, q_scale: float,
+             inv_tau: float) -> torch.Tensor:
+    """S <- diag(sigmoid(z_t)^inv_tau) S + k_t v_t^T, o_t = S^T (q_scale q_t) over the tokens of every
+    request of the step, from and to ``state`` float32 [slots, heads, dim, vdim].  ``proj`` [T, W] holds the
+    q, k (heads x dim) and v (heads x vdim) columns from ``q_off``, ``k_off``, ``v_off``; ``z`` float32
+    [T, heads * dim]; ``q_starts`` int32 [n + 1], ``seq_slots`` int32 [n].  Returns o float32 [T, heads * vdim]."""
+    _need(proj, "gla proj", ndim=2)
+    t, w = proj.shape
+    _need(z, "gla z", dtype=torch.float32, shape=(t, heads * dim))
+    _need(state, "gla state", dtype=torch.float32, ndim=4)
+    if tuple(state.shape[1:]) != (heads, dim, vdim):
+        raise KernelError(f"gla state: shape {tuple(state.shape)} is not [slots, {heads}, {dim}, {vdim}]")
+    _need(q_starts, "gla q_starts", dtype=torch.int32, ndim=1)
+    _need(seq_slots, "gla seq_slots", dtype=torch.int32, ndim=1)
+    n = seq_slots.shape[0]
+    if q_starts.shape[0] != n + 1:
+        raise KernelError("gla: q_starts must have one entry more than seq_slots")
+    out = torch.empty((t, heads * vdim), dtype=torch.float32, device=proj.device)
+    check(load().fsie_gla_scan(proj.data_ptr(), w, q_off, k_off, v_off, z.data_ptr(), state.data_ptr(), q_starts.data_ptr(),
+                               seq_slots.data_ptr(), n, out.data_ptr(), heads, dim, vdim, float(q_scale), float(inv_tau),
+                               state.shape[0], dtype_code(proj.dtype), _stream()))
+    return out
+
+
+# ---------------------------------------------------------------------------------------------
+# attention through a latent
+# ---------------------------------------------------------------------------------------------
+def latent_prep(proj: torch.Tensor, dq_off: int, q_rank: int, dkv_off: int, kv_rank: int, rot_dim: int, rot_pairs: int,
+                g_off: int, heads: int, q_weight: torch.Tensor, kv_weight: Optional[torch.Tensor], eps: float,
+                cos_sin: Optional[torch.Tensor], slots: Optional[torch.Tensor] = None,
+                k_pool: Optional[torch.Tensor] = None, v_pool: Optional[torch.Tensor] = None):
+    """From the fused projection ``proj`` [T, W]: the normed query latent [T, q_rank] (type of ``proj``), the
+    sigmoid of the heads' gates (float32 [T, heads]) and, if pools are given, every token's cache row
+    [normed latent | key part with its first ``rot_pairs`` pairs of neighbours rotated | zeros] written at
+    ``slots`` into ``k_pool`` [units, 1, page, width] and (transposed) ``v_pool`` [units, 1, width, page]."""
+    _need(proj, "latent proj", ndim=2)
+    t, w = proj.shape
+    _need(q_weight, "latent q norm weight", dtype=torch.float32, shape=(q_rank,))
+    width = page_size = pool_slots = 0
+    if k_pool is not None:
+        _need(k_pool, "k_pool", dtype=proj.dtype, ndim=4)
+        units, kvh, page_size, width = k_pool.shape
+        _need(v_pool, "v_pool", dtype=proj.dtype, shape=(units, kvh, width, page_size))
+        if kvh != 1:
+            raise KernelError("latent_prep: the latent cache has one kv head")
+        _need(slots, "latent slots", dtype=torch.int32, shape=(t,))
+        _need(kv_weight, "latent kv norm weight", dtype=torch.float32, shape=(kv_rank,))
+        pool_slots = units * page_size
+        if rot_pairs:
+            _need(cos_sin, "latent cos/sin", dtype=torch.float32, shape=(t, rot_pairs, 2))
+    cq = torch.empty((t, q_rank), dtype=proj.dtype, device=proj.device)
+    gate = torch.empty((t, heads), dtype=torch.float32, device=proj.device)
+    check(load().fsie_latent_prep(proj.data_ptr(), w, dq_off, q_rank, dkv_off, kv_rank, rot_dim, rot_pairs, g_off, heads,
+                                  q_weight.data_ptr(), _ptr(kv_weight), float(eps), _ptr(cos_sin), cq.data_ptr(),
+                                  gate.data_ptr(), _ptr(slots), _ptr(k_pool), _ptr(v_pool), width, page_size, pool_slots, t,
+                                  dtype_code(proj.dtype), _stream()))
+    return cq, gate
+
+
+def rope_pairs(x: torch.Tensor, in_off: int, in_head_stride: int, out: torch.Tensor, out_off: int, out_head_stride: int,
+               heads: int, width: int, rot_pairs: int, out_width: int, cos_sin: Optional[torch.Tensor]) -> torch.Tensor:
+    """Of every token and head the run of ``width`` values at column ``in_off + h * in_head_stride`` of ``x``,
+    its first ``rot_pairs`` pairs of neighbours (2i, 2i + 1) rotated by ``cos_sin`` [T, rot_pairs, 2], written to
+    column ``out_off + h * out_head_stride`` of ``out`` and filled up with zeros to ``out_width`` values."""
+    _need(x, "rope_pairs x", ndim=2)
+    _need(out, "rope_pairs out", dtype=x.dtype, ndim=2)
+    t = x.shape[0]
+    if out.shape[0] != t:
+        raise KernelError("rope_pairs: x and out must have a row a token")
+    if rot_pairs:
+        _need(cos_sin, "rope_pairs cos/sin", dtype=torch.float32, shape=(t, rot_pairs, 2))
+    check(load().fsie_rope_pairs(x.data_ptr(), x.shape[1], in_off, in_head_stride, out.data_ptr(), out.shape[1], out_off,
+                                 out_head_stride, heads, width, rot_pairs, out_width, _ptr(cos_sin), t,
+                                 dtype_code(x.dtype), _stream()))
+    return out
+
+
+def head_gemm(x: torch.Tensor, x_off: int, x_head_stride: int, weight: torch.Tensor, out: torch.Tensor, out_off: int,
+              out_head_stride: int, gate: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``out[t, h, n] = (sum_k x[t, h, k] weight[h, n, k]) * gate[t, h]``: a matrix of its own for every head.
+    ``x`` [T, W] holds head h's K values from column ``x_off + h * x_head_stride``, ``out`` [T, V] receives its N
+    values from column ``out_off + h * out_head_stride``; ``weight`` [heads, N, K]; ``gate`` float32 [T, heads]."""
+    _need(x, "head_gemm x", ndim=2)
+    _need(weight, "head_gemm weight", dtype=x.dtype, ndim=3)
+    _need(out, "head_gemm out", dtype=x.dtype, ndim=2)
+    heads, n, k = weight.shape
+    t = x.shape[0]
+    if out.shape[0] != t:
+        raise KernelError("head_gemm: x and out must have a row a token")
+    if gate is not None:
+        _need(gate, "head_gemm gate", dtype=torch.float32, shape=(t, heads))
+    check(load().fsie_head_gemm(x.data_ptr(), x.shape[1], x_off, x_head_stride, weight.data_ptr(), out.data_ptr(),
+                                out.shape[1], out_off, out_head_stride, _ptr(gate), t, heads, n, k, dtype_code(x.dtype),
+                                _stream()))
     return out

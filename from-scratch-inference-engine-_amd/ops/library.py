@@ -53,22 +53,35 @@ _SIGNATURES = {
     "fsie_fragment_order_size": ([c_int, c_int], c_int64),
     "fsie_fragment_order": ([_P, _P, c_int, c_int, _P], c_int),
     "fsie_attention_scalar": ([_P, c_int64, _P, _P, _P, c_int, _P, c_int, _P, _P, c_int, c_int, c_int,
-                               c_int, c_int, c_float, c_int, _P], c_int),
+                               c_int, c_int, c_float, c_int, _P, _P], c_int),
     "fsie_attention_mfma": ([_P, c_int64, _P, _P, _P, c_int, _P, c_int, _P, _P, c_int, c_int, c_int,
-                             c_int, c_int, c_float, c_int, c_int, _P], c_int),
+                             c_int, c_int, c_float, c_int, c_int, _P, _P], c_int),
     "fsie_attention_mfma_qkv_ok": ([c_int, c_int], c_int),
     "fsie_attention_mfma_qkv": ([_P, c_int, c_int, _P, _P, _P, _P, _P, c_int64, _P, c_int, _P, c_int, _P, _P, c_int,
                                  c_int, c_int, c_int, c_int, c_float, c_int, _P], c_int),
     "fsie_attention_mfma_max_waves": ([c_int], c_int),
     "fsie_attention_mfma_lds_ok": ([c_int, c_int], c_int),
     "fsie_attention_mfma_lds": ([_P, c_int64, _P, _P, _P, c_int, _P, _P, c_int, _P, c_int, c_int, c_int, c_int, c_int,
-                                 c_float, _P], c_int),
+                                 c_float, _P, _P], c_int),
     "fsie_attention_mfma_tiles": ([c_int, c_int], c_int),
-    "fsie_attention_merge": ([_P, _P, c_int, _P, c_int, c_int, c_int, _P], c_int),
+    "fsie_attention_merge": ([_P, _P, c_int, _P, c_int, c_int, c_int, _P, _P], c_int),
     "fsie_attention_scalar_tile_tokens": ([c_int, c_int], c_int),
     "fsie_static_scratch_bytes": ([], c_int64),
     "fsie_attention_split_static": ([_P, c_int64, _P, _P, _P, c_int, _P, c_int, _P, c_int, c_int, _P, c_int, c_int,
                                      c_int, c_int, c_int, c_float, c_int, c_int, c_int, _P], c_int),
+    "fsie_gated_act": ([_P, _P, c_int, c_int, c_int, c_int, _P], c_int),
+    "fsie_gemm_mfma_wide_gated": ([_P, _P, _P, c_int, c_int, c_int, c_int, c_int, c_int, c_int, _P], c_int),
+    "fsie_sandwich_norm": ([_P, _P, _P, c_float, _P, c_float, _P, _P, c_int, c_int, c_int, c_int, c_int, c_int, _P], c_int),
+    "fsie_gated_headnorm": ([_P, _P, c_int64, _P, _P, c_int, c_int, c_int, c_float, c_int, c_int, _P], c_int),
+    "fsie_softcap": ([_P, c_int64, c_float, _P], c_int),
+    "fsie_gla_scan": ([_P, c_int64, c_int, c_int, c_int, _P, _P, _P, _P, c_int, _P, c_int, c_int, c_int, c_float, c_float,
+                       c_int, c_int, _P], c_int),
+    "fsie_latent_prep": ([_P, c_int64, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, _P, _P, c_float, _P, _P, _P,
+                          _P, _P, _P, c_int, c_int, c_int64, c_int, c_int, _P], c_int),
+    "fsie_rope_pairs": ([_P, c_int64, c_int, c_int, _P, c_int64, c_int, c_int, c_int, c_int, c_int, c_int, _P, c_int, c_int,
+                         _P], c_int),
+    "fsie_head_gemm": ([_P, c_int64, c_int, c_int, _P, _P, c_int64, c_int, c_int, _P, c_int, c_int, c_int, c_int, c_int, _P],
+                       c_int),
     "fsie_sample": ([_P, c_int, c_int, _P, _P, _P, _P, _P, _P], c_int),
 }
 

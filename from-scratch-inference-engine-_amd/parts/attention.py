@@ -315,12 +315,50 @@ class AttentionPlanner:
         }
 
 
+def paged_attention(q: torch.Tensor, q_stride: int, cache, plan, n_heads: int, n_kv: int, head_dim: int,
+                    window: Optional[int], scale: float, n_tokens: int, sinks: Optional[torch.Tensor] = None,
+                    share_keys: bool = True) -> torch.Tensor:
+    """Causal attention of a step's queries over the paged cache, by the work items of ``plan`` (an
+    ``AttentionPlanner``'s): [n_tokens, n_heads * head_dim] in the queries' type.  ``q``: rows of ``q_stride``
+    values whose first n_heads * head_dim are the heads' queries; the keys and values of the step's own
+    tokens are in the cache already.  ``sinks`` (float32 [n_heads] or None): a term exp(sinks[h]) more in the
+    denominator of head h's softmax.  Every mixer whose cache is pages of keys and values calls this."""
+    out = torch.empty((n_tokens, n_heads * head_dim), dtype=q.dtype, device=q.device)
+    partials = None
+    if plan.n_partial:
+        partials = torch.empty((plan.n_partial * n_heads * (head_dim + 2),), dtype=torch.float32, device=q.device)
+    args = (partials, n_heads, n_kv, head_dim, window, scale, n_tokens)
+    if plan.mfma:
+        if plan.n_small:
+            ops.attention_mfma(q, q_stride, cache.k_pool, cache.v_pool, cache.block_tables, plan.items,
+                               plan.n_small, out, *args, large=False, waves=plan.waves, sinks=sinks)
+        if plan.n_large and not plan.n_long and share_keys and ops.attention_mfma_lds_ok(head_dim, cache.page_size):
+            ops.attention_mfma_lds(q, q_stride, cache.k_pool, cache.v_pool, cache.block_tables,
+                                   plan.items[plan.n_small:], plan.groups, plan.n_groups, out, n_heads,
+                                   n_kv, head_dim, window, scale, n_tokens, sinks=sinks)
+        elif plan.n_large:
+            ops.attention_mfma(q, q_stride, cache.k_pool, cache.v_pool, cache.block_tables,
+                               plan.items[plan.n_small:], plan.n_large, out, *args, large=True, sinks=sinks)
+        if plan.n_long:
+            ops.attention_mfma(q, q_stride, cache.k_pool, cache.v_pool, cache.block_tables,
+                               plan.items[plan.n_small + plan.n_large:], plan.n_long, out, *args, large=True,
+                               waves=4, sinks=sinks)
+    else:
+        ops.attention_scalar(q, q_stride, cache.k_pool, cache.v_pool, cache.block_tables, plan.items,
+                             plan.n_small + plan.n_large, out, *args, sinks=sinks)
+    if plan.n_merges:
+        ops.attention_merge(partials, plan.merges, plan.n_merges, out, n_heads, head_dim, sinks=sinks)
+    return out
+
+
 @register_part("mixer", "gqa_attention")
 class GQAttention(Mixer):
     """q/k/v projections (one matrix, optional bias), optional norms of every q and k head,
     position encoding, causal attention with kv head = q head // (heads / kv heads) and scale
     1/sqrt(head_dim), output projection without bias (src/model/model.cpp:110-129,
     src/model/nn.cpp:151-226).  ``window`` = number of latest positions a query reads (None: all).
+    ``sink=True``: a learned number per head (parameter ``sink``) whose exponential joins the softmax's
+    denominator; it has no key and no value.
 
     What happens between the projection and attention, in this order: bias, ``q_norm`` / ``k_norm``
     (a norm as wide as a head, applied to every head through ``Norm.plain``; None: none), the
@@ -345,7 +383,7 @@ class GQAttention(Mixer):
 
     def __init__(self, hidden_size: int, n_heads: int, n_kv_heads: int, head_dim: int, qkv_bias: bool,
                  position: PositionEncoding, window: Optional[int] = None, q_norm: Optional[Norm] = None,
-                 k_norm: Optional[Norm] = None):
+                 k_norm: Optional[Norm] = None, sink: bool = False):
         if n_heads % n_kv_heads:
             raise ValueError(f"attention: heads {n_heads} must be a multiple of kv heads {n_kv_heads}")
         if head_dim > 256:
@@ -359,6 +397,8 @@ class GQAttention(Mixer):
         self.o = Linear(self.q_dim, hidden_size)
         self.scale = 1.0 / math.sqrt(head_dim)
         self._planner: Optional[AttentionPlanner] = None
+        self.has_sink = bool(sink)
+        self.sink: Optional[torch.Tensor] = None
 
     def sub_parts(self) -> Dict[str, Part]:
         parts: Dict[str, Part] = {"position": self.position}
@@ -374,6 +414,8 @@ class GQAttention(Mixer):
                  "o_weight": ParamDecl((self.hidden_size, self.q_dim))}
         if self.qkv.has_bias:
             decls["qkv_bias"] = ParamDecl((self.q_dim + 2 * self.kv_dim,), "vector", "bias")
+        if self.has_sink:
+            decls["sink"] = ParamDecl((self.n_heads,), "vector", "bias")
         return decls
 
     qkv_weight = property(lambda s: s.qkv.weight, lambda s, t: setattr(s.qkv, "weight", t))
@@ -409,7 +451,7 @@ class GQAttention(Mixer):
     def _from_sums(self, x: torch.Tensor, ctx, cache, plan, table) -> Optional[torch.Tensor]:
         """Attention of a step of one token a request straight from the q/k/v product's partial sums
         (None: not such a step, or the kernels do not take the sizes)."""
-        if not (self.finish_qkv_in_attention and table is not None and cache.writes and plan.mfma and plan.single
+        if not (self.finish_qkv_in_attention and self.sink is None and table is not None and cache.writes and plan.mfma and plan.single
                 and plan.n_small and not plan.n_large and not plan.n_long and x.dtype == torch.bfloat16
                 and ops.attention_mfma_qkv_ok(self.head_dim, cache.page_size)):
             return None
@@ -475,32 +517,6 @@ class GQAttention(Mixer):
         if out is not None:
             return self.o.for_residual(out, ctx)
         qkv = self._project_rotate_store(x, ctx, cache, table)
-        t = x.shape[0]
-        out = torch.empty((t, self.q_dim), dtype=x.dtype, device=x.device)
-        partials = None
-        if plan.n_partial:
-            partials = torch.empty((plan.n_partial * self.n_heads * (self.head_dim + 2),), dtype=torch.float32,
-                                   device=x.device)
-        args = (partials, self.n_heads, self.n_kv, self.head_dim, self.window, self.scale, t)
-        if plan.mfma:
-            if plan.n_small:
-                ops.attention_mfma(qkv, qkv.shape[1], cache.k_pool, cache.v_pool, cache.block_tables, plan.items,
-                                   plan.n_small, out, *args, large=False, waves=plan.waves)
-            if plan.n_large and not plan.n_long and self.share_keys and ops.attention_mfma_lds_ok(self.head_dim,
-                                                                                                   cache.page_size):
-                ops.attention_mfma_lds(qkv, qkv.shape[1], cache.k_pool, cache.v_pool, cache.block_tables,
-                                       plan.items[plan.n_small:], plan.groups, plan.n_groups, out, self.n_heads,
-                                       self.n_kv, self.head_dim, self.window, self.scale, t)
-            elif plan.n_large:
-                ops.attention_mfma(qkv, qkv.shape[1], cache.k_pool, cache.v_pool, cache.block_tables,
-                                   plan.items[plan.n_small:], plan.n_large, out, *args, large=True)
-            if plan.n_long:
-                ops.attention_mfma(qkv, qkv.shape[1], cache.k_pool, cache.v_pool, cache.block_tables,
-                                   plan.items[plan.n_small + plan.n_large:], plan.n_long, out, *args, large=True,
-                                   waves=4)
-        else:
-            ops.attention_scalar(qkv, qkv.shape[1], cache.k_pool, cache.v_pool, cache.block_tables, plan.items,
-                                 plan.n_small + plan.n_large, out, *args)
-        if plan.n_merges:
-            ops.attention_merge(partials, plan.merges, plan.n_merges, out, self.n_heads, self.head_dim)
+        out = paged_attention(qkv, qkv.shape[1], cache, plan, self.n_heads, self.n_kv, self.head_dim, self.window,
+                              self.scale, x.shape[0], sinks=self.sink, share_keys=self.share_keys)
         return self.o.for_residual(out, ctx)

@@ -46,13 +46,16 @@ class HiddenState:
     """The residual stream of a step: ``residual`` float32 [T, H] and a pending ``delta`` that has
     not been added yet: [T, H] in the compute dtype, or (only if every norm of the model sets
     ``adds_partial_sums``, which the step's context then says in ``partial_sums_ok``) float32
-    [S, T, H], partial sums of a matrix product to be added in order."""
+    [S, T, H], partial sums of a matrix product to be added in order.  ``delta_norm``: a norm that the
+    pending delta goes through before it is added (a layer that also norms its sublayers' outputs), or
+    None; the norm that folds the delta in applies it in the same pass."""
 
-    __slots__ = ("residual", "delta")
+    __slots__ = ("residual", "delta", "delta_norm")
 
-    def __init__(self, residual: torch.Tensor, delta: Optional[torch.Tensor] = None):
+    def __init__(self, residual: torch.Tensor, delta: Optional[torch.Tensor] = None, delta_norm=None):
         self.residual = residual
         self.delta = delta
+        self.delta_norm = delta_norm
 
 
 class Part:

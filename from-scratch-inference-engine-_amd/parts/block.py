@@ -2,7 +2,7 @@
 
 from __future__ import annotations
 
-from typing import Dict
+from typing import Dict, Optional
 
 from .base import Block, FeedForward, HiddenState, Mixer, Norm, Part, register_part
 
@@ -26,3 +26,33 @@ class PreNormBlock(Block):
         hidden.delta = self.mixer.forward(x, ctx, cache)
         x = self.ffn_norm(hidden, ctx.compute_dtype)
         hidden.delta = self.ffn.forward(x, ctx)
+
+
+@register_part("block", "sandwich_norm")
+class SandwichNormBlock(Block):
+    """A norm before and after every sublayer: x += post1(mixer(norm1(x))); x += post2(ffn(norm2(x))).
+    A sublayer's output stays pending in the hidden state together with its post norm; the norm that reads
+    the stream next (this block's second, the next block's first, the model's last) runs the post norm,
+    the sum and itself in one pass.  ``ffn=None``: the layer has no feed-forward (and no norms for it)."""
+
+    graph_safe = True
+
+    def __init__(self, mixer_norm: Norm, mixer: Mixer, mixer_post_norm: Norm, ffn_norm: Optional[Norm] = None,
+                 ffn: Optional[FeedForward] = None, ffn_post_norm: Optional[Norm] = None):
+        if (ffn is None) != (ffn_norm is None) or (ffn is None) != (ffn_post_norm is None):
+            raise ValueError("sandwich_norm block: a feed-forward comes with both of its norms, or none of the three")
+        self.mixer_norm, self.mixer, self.mixer_post_norm = mixer_norm, mixer, mixer_post_norm
+        self.ffn_norm, self.ffn, self.ffn_post_norm = ffn_norm, ffn, ffn_post_norm
+
+    def sub_parts(self) -> Dict[str, Part]:
+        parts = {"mixer_norm": self.mixer_norm, "mixer": self.mixer, "mixer_post_norm": self.mixer_post_norm}
+        if self.ffn is not None:
+            parts.update(ffn_norm=self.ffn_norm, ffn=self.ffn, ffn_post_norm=self.ffn_post_norm)
+        return parts
+
+    def forward(self, hidden: HiddenState, ctx, cache) -> None:
+        x = self.mixer_norm(hidden, ctx.compute_dtype)
+        hidden.delta, hidden.delta_norm = self.mixer.forward(x, ctx, cache), self.mixer_post_norm
+        if self.ffn is not None:
+            x = self.ffn_norm(hidden, ctx.compute_dtype)
+            hidden.delta, hidden.delta_norm = self.ffn.forward(x, ctx), self.ffn_post_norm

@@ -2,7 +2,7 @@
 
 from __future__ import annotations
 
-from typing import Dict
+from typing import Dict, Optional
 
 import torch
 
@@ -31,12 +31,16 @@ class TokenEmbedding(Part):
 
 class LMHead(Part):
     """logits = x . W^T in float32, no bias (src/model/model.cpp:144-148).  With tied embeddings
-    its weight is bound to the embedding table."""
+    its weight is bound to the embedding table.  ``softcap`` (a positive number): the logits become
+    softcap * tanh(logits / softcap)."""
 
     kind = "lm_head"
     graph_safe = True
 
-    def __init__(self, hidden_size: int, vocab_size: int):
+    def __init__(self, hidden_size: int, vocab_size: int, softcap: Optional[float] = None):
+        if softcap is not None and not softcap > 0:
+            raise ValueError(f"lm head: softcap {softcap} must be positive")
+        self.softcap = None if softcap is None else float(softcap)
         self.linear = Linear(hidden_size, vocab_size)
         self.vocab_size, self.hidden_size = vocab_size, hidden_size
 
@@ -58,4 +62,5 @@ class LMHead(Part):
         return self.linear.drop_copy()
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
-        return self.linear(x, out_dtype=torch.float32)
+        logits = self.linear(x, out_dtype=torch.float32)
+        return logits if self.softcap is None else ops.softcap(logits, self.softcap)

@@ -12,16 +12,20 @@ from ..ops.functions import GEMM_MFMA_SKINNY_BEST_M
 from .linear import Linear
 
 
+@register_part("feed_forward", "gated")
 @register_part("feed_forward", "swiglu")
 class SwiGLU(FeedForward):
-    """down(silu(gate(x)) * up(x)), no biases (src/model/model.cpp:134-138).  gate and up are one
+    """down(act(gate(x)) * up(x)), no biases, act = SiLU (src/model/model.cpp:134-138) unless ``activation``
+    names another one the kernels know ("gelu_tanh").  gate and up are one
     matrix [2I, H] with their rows interleaved (gate_0, up_0, gate_1, up_1, ...): x is read once,
     and the lane that holds gate_j also holds up_j, so that for a few rows (decoding) SiLU*up
     happens in the product's epilogue and the [T, 2I] intermediate never reaches memory."""
 
     graph_safe = True
 
-    def __init__(self, hidden_size: int, intermediate_size: int):
+    def __init__(self, hidden_size: int, intermediate_size: int, activation: str = "silu"):
+        ops.gate_act_code(activation)  # refuses a name the kernels do not know
+        self.activation = activation
         self.hidden_size = hidden_size
         self.intermediate_size = intermediate_size
         self.gate_up = Linear(hidden_size, 2 * intermediate_size)
@@ -65,14 +69,15 @@ class SwiGLU(FeedForward):
                 and self.gate_up.wide_takes(m, 1, gate_up=True)):
             # from the fragment-ordered copy at any number of rows up to 64, and up to 128 where the
             # kernel has the launch shape for it: SiLU*up in the product's epilogue
-            act = ops.gemm_mfma_wide_swiglu(x, self.gate_up.streamed)
+            act = ops.gemm_mfma_wide_swiglu(x, self.gate_up.streamed, act=self.activation)
         elif (x.dtype == torch.bfloat16 and 3 <= m <= GEMM_MFMA_SKINNY_BEST_M and self.hidden_size % 128 == 0
                 and self.gate_up.out_features % 4 == 0 and self.gate_up.out_features // 64 >= ops.compute_units()):
             # three rows and more of a matrix that gives every compute unit a workgroup: the kernel that
             # shares x through LDS (one or two rows, and small matrices, are faster in the other)
-            act = ops.gemm_mfma_wide_swiglu(x, self.gate_up.weight)
+            act = ops.gemm_mfma_wide_swiglu(x, self.gate_up.weight, act=self.activation)
         elif x.dtype == torch.bfloat16 and m <= GEMM_MFMA_SKINNY_BEST_M and self.hidden_size % 8 == 0:
-            act = ops.gemm_mfma_skinny(x, self.gate_up.weight, epilogue="swiglu")
+            act = ops.gemm_mfma_skinny(x, self.gate_up.weight,
+                                       epilogue="swiglu" if self.activation == "silu" else "geglu_tanh")
         else:
-            act = ops.swiglu(self.gate_up(x))
+            act = ops.swiglu(self.gate_up(x), act=self.activation)
         return self.down.for_residual(act, ctx)

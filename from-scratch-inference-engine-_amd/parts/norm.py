@@ -14,26 +14,45 @@ from .base import HiddenState, Norm, ParamDecl, register_part
 class RMSNorm(Norm):
     """y = (x * rsqrt(mean(x^2) + eps)) * w with x = residual + pending delta, all in float32;
     eps inside the square root, the weight multiplied last, plain w (the reference's rms_norm,
-    src/model/nn.cpp:45-72, which sums in float64)."""
+    src/model/nn.cpp:45-72, which sums in float64).  ``unit_offset=True``: the checkpoint tensor is the
+    factor less one, so the factor is 1 + w (the one is added in float32 when the weights are loaded).
+    Where the pending delta has a norm of its own to go through first (``HiddenState.delta_norm``, another
+    ``RMSNorm``), that norm, the sum and this norm are one kernel."""
 
     adds_partial_sums = True
 
     graph_safe = True
 
-    def __init__(self, hidden_size: int, eps: float):
+    def __init__(self, hidden_size: int, eps: float, unit_offset: bool = False):
         self.hidden_size = hidden_size
         self.eps = float(eps)
+        self.unit_offset = bool(unit_offset)
         self.weight = None
+        self._offset_added = False
 
     def param_decls(self) -> Dict[str, ParamDecl]:
-        return {"weight": ParamDecl((self.hidden_size,), "vector", "norm")}
+        # (an offset from one is drawn like a bias by the random-weights mode: small, centred on zero)
+        return {"weight": ParamDecl((self.hidden_size,), "vector", "bias" if self.unit_offset else "norm")}
+
+    def prepare(self, device, compute_dtype) -> None:
+        if self.unit_offset and not self._offset_added and self.weight is not None:
+            self.weight = self.weight + 1.0
+            self._offset_added = True
 
     def __call__(self, hidden: HiddenState, out_dtype: torch.dtype) -> torch.Tensor:
-        delta, hidden.delta = hidden.delta, None
+        delta, post = hidden.delta, hidden.delta_norm
+        hidden.delta = hidden.delta_norm = None
+        if delta is not None and post is not None:
+            return ops.sandwich_norm(hidden.residual, delta, post.weight, post.eps, self.weight, self.eps, out_dtype,
+                                     write_back=True)
         return ops.rmsnorm(hidden.residual, self.weight, self.eps, out_dtype, delta=delta,
                            write_back=delta is not None)
 
     def rows(self, hidden: HiddenState, rows: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
+        if hidden.delta is not None and hidden.delta_norm is not None:
+            post = hidden.delta_norm
+            return ops.sandwich_norm(hidden.residual, hidden.delta, post.weight, post.eps, self.weight, self.eps,
+                                     out_dtype, rows=rows)
         return ops.rmsnorm(hidden.residual, self.weight, self.eps, out_dtype, delta=hidden.delta, rows=rows)
 
     def plain(self, x: torch.Tensor, out=None) -> torch.Tensor:

@@ -16,11 +16,16 @@ class RotaryEncoding(PositionEncoding):
     """Rotate-half RoPE over ``rotary_dim`` (default: the whole head): pair (i, i + rotary_dim/2),
     frequency theta^(-2i/rotary_dim), angle = position * frequency in float64
     (src/model/nn.cpp:110-149).  Where the whole head rotates it also offers the step's table of
-    cosines and sines, from which a mixer's own kernels rotate."""
+    cosines and sines, from which a mixer's own kernels rotate.  ``layout="interleaved"``: the pairs are
+    neighbours (2i, 2i + 1) instead, the frequencies the same; ``table`` gives a mixer the step's cosines
+    and sines for its own kernels, ``rotate`` turns the first ``rotary_dim`` values of every q and k head."""
 
     graph_safe = True
 
-    def __init__(self, head_dim: int, theta: float, rotary_dim: Optional[int] = None):
+    def __init__(self, head_dim: int, theta: float, rotary_dim: Optional[int] = None, layout: str = "half"):
+        if layout not in ("half", "interleaved"):
+            raise ValueError(f"rope: unknown layout '{layout}' (half or interleaved)")
+        self.layout = layout
         self.head_dim = head_dim
         self.theta = float(theta)
         self.rotary_dim = head_dim if rotary_dim is None else rotary_dim
@@ -43,9 +48,14 @@ class RotaryEncoding(PositionEncoding):
         return table
 
     def rotation_table(self, head_dim, ctx):
-        return self.table(ctx) if self.rotary_dim == head_dim else None
+        return self.table(ctx) if self.rotary_dim == head_dim and self.layout == "half" else None
 
     def rotate(self, qkv, n_heads, n_kv, head_dim, ctx) -> None:
+        if self.layout == "interleaved":
+            # (a lane reads its neighbour's value: from a copy, so that nobody reads what another has written)
+            ops.rope_pairs(qkv.clone(), 0, head_dim, qkv, 0, head_dim, n_heads + n_kv, head_dim, self.rotary_dim // 2,
+                           head_dim, self.table(ctx))
+            return
         cos_sin = self.table(ctx) if self.rotary_dim == head_dim and head_dim % 8 == 0 else None
         ops.rope_kv_write(qkv, ctx.positions, n_heads, n_kv, head_dim, self.inv_freq, cos_sin=cos_sin)
 

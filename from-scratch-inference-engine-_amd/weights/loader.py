@@ -220,6 +220,18 @@ class CheckpointFiles:
         return self._where[name].get(name)
 
 
+def tensor_shapes(path) -> Dict[str, Tuple[int, ...]]:
+    """Name -> shape of every tensor of a .safetensors file or a model folder (the headers only are read);
+    nothing if the folder holds no weights."""
+    import os
+
+    try:
+        f = CheckpointFiles(path) if os.path.isdir(path) else SafetensorsFile(path)
+    except (OSError, WeightsError):
+        return {}
+    return {n: tuple(f.shape(n)) for n in f.names()}
+
+
 def load_weights(path, bindings: Sequence[ParamBinding], compute_dtype: torch.dtype, device,
                  ignore_unexpected: Sequence[str] = ()) -> int:
     """Check ``path`` (a .safetensors file, or a model folder: see ``CheckpointFiles``) against
