@@ -129,7 +129,8 @@ def run_trace(model_dir, dtype: str, steps, max_tokens: int, out_dir, timeout: i
         raise AssertionError(f"trace_run failed ({proc.returncode}):\n{proc.stdout[-2000:]}\n{proc.stderr[-4000:]}")
     done = [line for line in proc.stdout.splitlines() if line.startswith("done ")]
     assert [d.split()[1] for d in done] == [str(s["step"]) for s in steps], "one 'done <step>' line per step, in order"
-    vocab = json.loads((Path(model_dir) / "config.json").read_text())["vocab_size"]
+    raw = json.loads((Path(model_dir) / "config.json").read_text())
+    vocab = raw["vocab_size"] if "vocab_size" in raw else raw["vocab"]
     out = {}
     for s in steps:
         f = out_dir / f"{s['step']}.f32"
