@@ -229,6 +229,100 @@ def other_workload(args, cfg, model, shape_name, layers, full_layers, page, fill
     return 0
 
 
+def gilozen_shape(width: int, ff: int, layers: int, vocab: int) -> dict:
+    """A Gilozen configuration of real layer sizes: two layers of gated linear attention, then one of attention
+    through a latent, over and over; every second attention layer reads the cache of the one before it."""
+    heads = width // 128
+    gla = {"heads": heads // 2, "dim": 128, "vdim": 256, "tau": 16.0, "a_rank": 64}
+    latent = {"heads": heads, "dim": 64, "rot_dim": 64, "vdim": 128, "kv_rank": 192, "q_rank": width // 2 + 256,
+              "scale": 128 ** -0.5, "rot": {"base": 500000.0, "dims": 64}}
+    out, last_latent, borrow = [], None, False
+    for i in range(layers):
+        if i % 3 == 2:
+            m = dict(latent)
+            if borrow and last_latent is not None:
+                m["kv_from"] = last_latent
+            else:
+                last_latent = i
+            borrow = not borrow
+            out.append({"type": "latent_attention", "mixer": m, "mlp": {"kind": "dense", "ff": ff}})
+        else:
+            out.append({"type": "gla", "mixer": dict(gla), "mlp": {"kind": "dense", "ff": ff}})
+    return {"architecture": "Gilozen", "width": width, "vocab": vocab, "norm": {"eps": 1e-5}, "logit_softcap": 30.0,
+            "layers": out}
+
+
+DESIGN_SIZES = {"2048": (2048, 8192, 9, 32000), "4096": (4096, 14336, 9, 32000)}  # width, ff, layers, vocab
+
+
+def design_comparison(args) -> int:
+    """--workload gilozen: prefill (one prompt of 2,048 tokens in one step) and decode (batches of 8 and 64 at a
+    context of 512, from captured graphs) of Gilozen at two real layer sizes with random weights, beside a Qwen2
+    model of the same width, feed-forward, layers and vocabulary (grouped-query attention, 128 values a head, four
+    query heads a key/value head) through the same step function.  One JSON line."""
+    import torch
+
+    from from_scratch_inference_engine_amd.engine.context import StepEntry
+    from from_scratch_inference_engine_amd.engine.model import Model, Runner
+    from from_scratch_inference_engine_amd.models import parse_config
+
+    dtype = "bfloat16" if args.dtype == "bf16" else "float32"
+    gen = torch.Generator().manual_seed(0)
+    results = {}
+    phases = args.design_phases.split(",")
+    for size in args.design_sizes.split(","):
+        width, ff, layers, vocab = DESIGN_SIZES[size]
+        qwen = {"architectures": ["Qwen2ForCausalLM"], "model_type": "qwen2", "hidden_size": width,
+                "num_hidden_layers": layers, "num_attention_heads": width // 128, "num_key_value_heads": width // 512,
+                "head_dim": 128, "intermediate_size": ff, "vocab_size": vocab, "rope_theta": 500000.0,
+                "rms_norm_eps": 1e-5, "tie_word_embeddings": False, "max_position_embeddings": 8192}
+        for name, raw in (("gilozen", gilozen_shape(width, ff, layers, vocab)), ("qwen2", qwen)):
+            model = Model.from_random(parse_config(raw), seed=0, dtype=dtype)
+            runner = Runner(model, page_size=16, num_pages=64 * 40 + 160, max_requests=64)
+            row = {"weights_gb": model.weight_bytes / 1e9}
+            times = []
+            for rep in range(4 if "prefill" in phases else 0):
+                rc = runner.manager.open(f"p{rep}")
+                ids = torch.randint(0, vocab, (2048,), generator=gen).tolist()
+                torch.cuda.synchronize()
+                t = time.perf_counter()
+                runner.step([StepEntry(rc, ids, [2047])])
+                torch.cuda.synchronize()
+                times.append(time.perf_counter() - t)
+                runner.manager.close(rc)
+            if times:
+                row["prefill_2048_ms"] = min(times[1:]) * 1e3
+                row["prefill_tok_s"] = 2048 / min(times[1:])
+            for batch in ((8, 64) if "decode" in phases else ()):
+                caches = [runner.manager.open(f"d{batch}.{i}") for i in range(batch)]
+                for c in caches:
+                    runner.step([StepEntry(c, torch.randint(0, vocab, (512,), generator=gen).tolist(), [])])
+                step = lambda: runner.step([StepEntry(c, [7], [0]) for c in caches], keep=False)
+                for _ in range(args.warmup):
+                    step()
+                torch.cuda.synchronize()
+                t = time.perf_counter()
+                for _ in range(args.steps):
+                    step()
+                torch.cuda.synchronize()
+                dt = (time.perf_counter() - t) / args.steps
+                row[f"decode_b{batch}_ms"] = dt * 1e3
+                row[f"decode_b{batch}_tok_s"] = batch / dt
+                row[f"decode_b{batch}_weights_gb_s"] = model.weight_bytes / dt / 1e9
+                for c in caches:
+                    runner.manager.close(c)
+            results.setdefault(size, {})[name] = row
+            print(f"[bench] width {width} {name}: " + ", ".join(f"{k} {v:.3f}" for k, v in row.items()), file=sys.stderr, flush=True)
+            del runner, model
+            torch.cuda.empty_cache()
+    print(json.dumps({"metric": "Gilozen beside Qwen2 at equal sizes: prefill tok/s @ 2,048 tokens, decode tok/s @ batch 8 and 64, context 512",
+                      "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "dtype": args.dtype,
+                      "data": "synthetic: random weights N(0,0.02), uniform random token ids",
+                      "sizes": {k: dict(zip(("width", "ff", "layers", "vocab"), DESIGN_SIZES[k])) for k in results},
+                      "results": results}))
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -246,11 +340,13 @@ def main() -> int:
     ap.add_argument("--no-tune", action="store_true", help="leave the library's kernel choice for prefill to its heuristic")
     ap.add_argument("--no-streamed-copies", action="store_true",
                     help="do not keep the large weights a second time in the order of the matrix instruction's fragments")
-    ap.add_argument("--workload", choices=["decode", "mixed", "long-prefill"], default="decode",
+    ap.add_argument("--design-sizes", default="2048,4096", help="--workload gilozen: widths to run (2048, 4096)")
+    ap.add_argument("--design-phases", default="prefill,decode", help="--workload gilozen: what to time (for a trace of one phase)")
+    ap.add_argument("--workload", choices=["decode", "mixed", "long-prefill", "gilozen"], default="decode",
                     help="decode: the default run.  mixed: --requests prompts of --min-prompt to --max-prompt tokens, "
                          "--outputs tokens each, through the scheduler (made for --shape 14b).  "
                          "long-prefill: one prompt of --prefill-tokens tokens in portions of the token budget "
-                         "(made for --shape 32b)")
+                         "(made for --shape 32b).  gilozen: the Gilozen design beside Qwen2 at equal layer sizes")
     ap.add_argument("--requests", type=int, default=32)
     ap.add_argument("--min-prompt", type=int, default=128)
     ap.add_argument("--max-prompt", type=int, default=4096)
@@ -276,6 +372,8 @@ def main() -> int:
         enable_library_tuning()  # the first prefill times the library's kernels for its shapes
         fill_rows = padded_tokens  # and steps that are not decode steps are filled up to the timed row counts
 
+    if args.workload == "gilozen":
+        return design_comparison(args)
     shape_name, shape = SHAPES[args.shape]
     raw = dict(shape)
     full_layers = raw["num_hidden_layers"]

@@ -12,24 +12,28 @@
 
 namespace {
 
-constexpr int kGlaThreads = 256;  // four waves: wave w owns the key channels [w ROWS, (w + 1) ROWS), lane = value column
+constexpr int kGlaWaves = 16;  // wave w owns the key channels [w ROWS, (w + 1) ROWS), lane = value column
+constexpr int kGlaThreads = 64 * kGlaWaves;
 constexpr int kGlaCols = 64;
 
 // log(sigmoid(z)) without overflow: min(z, 0) - log(1 + exp(-|z|))
 __device__ __forceinline__ float log_sigmoid(float z) { return fminf(z, 0.f) - log1pf(expf(-fabsf(z))); }
 
-// grid = (requests of the step, heads, ceil(vdim / 64)).  A workgroup keeps its [dim][64] slice of the
-// state in registers (ROWS values a thread), takes the portion's tokens in tiles of TT through LDS
-// (q scaled, k, and the decays already as numbers in (0, 1)), and adds the four waves' shares of every
-// o_t through LDS in the order of the waves.
+// grid = (requests of the step, heads, ceil(vdim / 64)).  A workgroup of sixteen waves keeps its [dim][64]
+// slice of the state in registers (ROWS values a thread: few, so that a token costs a wave only 3 ROWS
+// instructions and the sixteen waves hide each other's waits), takes the portion's tokens in tiles of TT
+// through LDS (q scaled, k, and the decays already as numbers in (0, 1), read by every lane of a wave at
+// the same address), and adds the waves' shares of every o_t through LDS in the order of the waves.
 template <typename T, int ROWS, int TT>
 __global__ __launch_bounds__(kGlaThreads) void gla_scan_kernel(
     const T* __restrict__ proj, int64_t proj_stride, int q_off, int k_off, int v_off, const float* __restrict__ z,
     float* __restrict__ state, const int32_t* __restrict__ q_starts, const int32_t* __restrict__ seq_slots,
     float* __restrict__ out, int heads, int dim, int vdim, float q_scale, float inv_tau, int n_slots) {
-    constexpr int DP = 4 * ROWS;
-    __shared__ float qs[TT][DP], ks[TT][DP], as[TT][DP];
-    __shared__ float part[4][TT][kGlaCols];
+    constexpr int DP = kGlaWaves * ROWS;
+    constexpr int VW = ROWS % 4 == 0 ? 4 : 2;  // values of a shared-memory load (ROWS is 2, 4, 8 or 16)
+    typedef float Vec __attribute__((ext_vector_type(VW)));
+    __shared__ __attribute__((aligned(16))) float qs[TT][DP], ks[TT][DP], as[TT][DP];
+    __shared__ float part[kGlaWaves][TT][kGlaCols];
     const int seq = blockIdx.x, h = blockIdx.y;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int col = blockIdx.z * kGlaCols + lane;
@@ -46,38 +50,65 @@ __global__ __launch_bounds__(kGlaThreads) void gla_scan_kernel(
         S[r] = (col_ok && i < dim) ? my_state[static_cast<int64_t>(i) * vdim] : 0.f;
     }
 
+    // The inputs of the next tile are asked for before the present one is worked on, and wait in registers:
+    // a tile costs a few hundred cycles of arithmetic, a trip to memory several times that.
+    constexpr int EPT = (TT * DP + kGlaThreads - 1) / kGlaThreads;
+    float rq[EPT], rk[EPT], rz[EPT], v_next[TT];
+    auto fetch = [&](int t0) {
+        const int nt = min(TT, hi - t0);
+#pragma unroll
+        for (int u = 0; u < EPT; ++u) {
+            const int e = tid + u * kGlaThreads;
+            const int tt = e / DP, i = e - tt * DP;
+            rq[u] = 0.f, rk[u] = 0.f, rz[u] = INFINITY;  // a channel or token that does not exist: q = k = 0, decay 1
+            if (tt < nt && i < dim) {
+                const T* row = proj + static_cast<int64_t>(t0 + tt) * proj_stride + h * dim + i;
+                rq[u] = to_float(row[q_off]);
+                rk[u] = to_float(row[k_off]);
+                rz[u] = z[(static_cast<int64_t>(t0 + tt) * heads + h) * dim + i];
+            }
+        }
+#pragma unroll
+        for (int tt = 0; tt < TT; ++tt) {
+            v_next[tt] = (tt < nt && col_ok)
+                             ? to_float(proj[static_cast<int64_t>(t0 + tt) * proj_stride + v_off + h * vdim + col]) : 0.f;
+        }
+    };
+    fetch(lo);
     for (int t0 = lo; t0 < hi; t0 += TT) {
         const int nt = min(TT, hi - t0);
         __syncthreads();  // the last tile's shares have been added up, its q, k and decays are no longer read
-        for (int e = tid; e < TT * DP; e += kGlaThreads) {
-            const int tt = e / DP, i = e - tt * DP;
-            float q = 0.f, k = 0.f, a = 1.f;
-            if (tt < nt && i < dim) {
-                const T* row = proj + static_cast<int64_t>(t0 + tt) * proj_stride + h * dim + i;
-                q = to_float(row[q_off]) * q_scale;
-                k = to_float(row[k_off]);
-                a = expf(inv_tau * log_sigmoid(z[(static_cast<int64_t>(t0 + tt) * heads + h) * dim + i]));
+#pragma unroll
+        for (int u = 0; u < EPT; ++u) {
+            const int e = tid + u * kGlaThreads;
+            if (e < TT * DP) {
+                const int tt = e / DP, i = e - tt * DP;
+                qs[tt][i] = rq[u] * q_scale;
+                ks[tt][i] = rk[u];
+                as[tt][i] = expf(inv_tau * log_sigmoid(rz[u]));
             }
-            qs[tt][i] = q;
-            ks[tt][i] = k;
-            as[tt][i] = a;
         }
         float v[TT];
 #pragma unroll
-        for (int tt = 0; tt < TT; ++tt) {
-            v[tt] = (tt < nt && col_ok)
-                        ? to_float(proj[static_cast<int64_t>(t0 + tt) * proj_stride + v_off + h * vdim + col]) : 0.f;
-        }
+        for (int tt = 0; tt < TT; ++tt) v[tt] = v_next[tt];
         __syncthreads();
+        if (t0 + TT < hi) fetch(t0 + TT);
 #pragma unroll
         for (int tt = 0; tt < TT; ++tt) {
             if (tt < nt) {  // the same for the whole workgroup
+                // this wave's channels of the token: every lane reads the same addresses, VW values a load
+                float a[ROWS], k[ROWS], q[ROWS];
+#pragma unroll
+                for (int r = 0; r < ROWS; r += VW) {
+                    *reinterpret_cast<Vec*>(&a[r]) = *reinterpret_cast<const Vec*>(&as[tt][wave * ROWS + r]);
+                    *reinterpret_cast<Vec*>(&k[r]) = *reinterpret_cast<const Vec*>(&ks[tt][wave * ROWS + r]);
+                    *reinterpret_cast<Vec*>(&q[r]) = *reinterpret_cast<const Vec*>(&qs[tt][wave * ROWS + r]);
+                }
                 float o = 0.f;
 #pragma unroll
                 for (int r = 0; r < ROWS; ++r) {
-                    const int i = wave * ROWS + r;
-                    S[r] = fmaf(as[tt][i], S[r], ks[tt][i] * v[tt]);
-                    o = fmaf(S[r], qs[tt][i], o);
+                    S[r] = fmaf(a[r], S[r], k[r] * v[tt]);
+                    o = fmaf(S[r], q[r], o);
                 }
                 part[wave][tt][lane] = o;
             }
@@ -87,8 +118,10 @@ __global__ __launch_bounds__(kGlaThreads) void gla_scan_kernel(
             const int tt = e >> 6, c = e & 63;
             const int cc = blockIdx.z * kGlaCols + c;
             if (cc < vdim) {
-                out[(static_cast<int64_t>(t0 + tt) * heads + h) * vdim + cc] =
-                    ((part[0][tt][c] + part[1][tt][c]) + part[2][tt][c]) + part[3][tt][c];
+                float o = part[0][tt][c];
+#pragma unroll
+                for (int w = 1; w < kGlaWaves; ++w) o += part[w][tt][c];
+                out[(static_cast<int64_t>(t0 + tt) * heads + h) * vdim + cc] = o;
             }
         }
     }
@@ -124,11 +157,11 @@ extern "C" int fsie_gla_scan(const void* proj, int64_t proj_stride, int q_off, i
     gla_scan_kernel<T, ROWS, TT><<<grid, kGlaThreads, 0, stream>>>(static_cast<const T*>(proj), proj_stride, q_off, k_off, \
                                                                    v_off, z, state, q_starts, seq_slots, out, heads, dim, \
                                                                    vdim, q_scale, inv_tau, n_slots)
-#define FSIE_GLA_BY_DIM(T)                          \
-    if (dim <= 32) FSIE_GLA_LAUNCH(T, 8, 16);       \
-    else if (dim <= 64) FSIE_GLA_LAUNCH(T, 16, 16); \
-    else if (dim <= 128) FSIE_GLA_LAUNCH(T, 32, 16); \
-    else FSIE_GLA_LAUNCH(T, 64, 8)
+#define FSIE_GLA_BY_DIM(T)                        \
+    if (dim <= 32) FSIE_GLA_LAUNCH(T, 2, 8);      \
+    else if (dim <= 64) FSIE_GLA_LAUNCH(T, 4, 8); \
+    else if (dim <= 128) FSIE_GLA_LAUNCH(T, 8, 8); \
+    else FSIE_GLA_LAUNCH(T, 16, 8)
     if (dtype == FSIE_F32) {
         FSIE_GLA_BY_DIM(float);
     } else {

@@ -52,6 +52,85 @@ __global__ __launch_bounds__(kThreads) void sandwich_norm_kernel(
     for (int j = threadIdx.x; j < hidden; j += kThreads) dst[j] = from_float<T>((row_buf[j] * scale) * weight[j]);
 }
 
+// Four consecutive elements: one 16-byte (float32) or 8-byte (bfloat16) access.
+__device__ __forceinline__ float4 load4(const float* p) { return *reinterpret_cast<const float4*>(p); }
+__device__ __forceinline__ float4 load4(const bf16_t* p) {
+    const uint2 w = *reinterpret_cast<const uint2*>(p);
+    return float4{__uint_as_float(w.x << 16), __uint_as_float(w.x & 0xffff0000u), __uint_as_float(w.y << 16),
+                  __uint_as_float(w.y & 0xffff0000u)};
+}
+__device__ __forceinline__ void store4(float* p, float4 v) { *reinterpret_cast<float4*>(p) = v; }
+__device__ __forceinline__ void store4(bf16_t* p, float4 v) {
+    uint2 w;
+    w.x = pack2_bf16(v.x, v.y);
+    w.y = pack2_bf16(v.z, v.w);
+    *reinterpret_cast<uint2*>(p) = w;
+}
+
+// The same for hidden % 4 == 0 and hidden <= 4 * THREADS * ITERS: a thread keeps its quads of the row in
+// registers, and every load of the row (stream, delta or partial sums, both weights) goes out before
+// anything waits.  Places past the end read the last quad again and are masked out of sums and stores.
+template <typename T, int ITERS, int THREADS>
+__global__ __launch_bounds__(THREADS) void sandwich_norm_vec_kernel(
+    float* __restrict__ residual, const T* __restrict__ delta, const float* __restrict__ post_weight, float post_eps,
+    const float* __restrict__ weight, float eps, T* __restrict__ out, const int32_t* __restrict__ rows, int hidden,
+    int write_back, int n_parts, int64_t part_stride) {
+    __shared__ float scratch[16];
+    const int r = blockIdx.x;
+    const int64_t row = rows ? rows[r] : r;
+    float* res = residual + row * hidden;
+    const T* del = n_parts ? nullptr : delta + row * hidden;
+    const float* parts = n_parts ? reinterpret_cast<const float*>(delta) + row * hidden : nullptr;
+    float4 y[ITERS], v[ITERS], wp[ITERS], w[ITERS];
+#pragma unroll
+    for (int it = 0; it < ITERS; ++it) {
+        const int j = min((it * THREADS + static_cast<int>(threadIdx.x)) * 4, hidden - 4);
+        v[it] = load4(res + j);
+        wp[it] = load4(post_weight + j);
+        w[it] = load4(weight + j);
+        if (del) {
+            y[it] = load4(del + j);
+        } else {
+            float4 a = load4(parts + j);
+#pragma unroll 4
+            for (int s = 1; s < n_parts; ++s) {
+                const float4 p = load4(parts + s * part_stride + j);
+                a.x += p.x, a.y += p.y, a.z += p.z, a.w += p.w;
+            }
+            y[it] = a;
+        }
+    }
+    float sum_sq = 0.f;
+#pragma unroll
+    for (int it = 0; it < ITERS; ++it) {
+        if ((it * THREADS + static_cast<int>(threadIdx.x)) * 4 < hidden)
+            sum_sq += y[it].x * y[it].x + y[it].y * y[it].y + y[it].z * y[it].z + y[it].w * y[it].w;
+    }
+    const float post_scale = 1.0f / sqrtf(block_sum(sum_sq, scratch) / static_cast<float>(hidden) + post_eps);
+    sum_sq = 0.f;
+#pragma unroll
+    for (int it = 0; it < ITERS; ++it) {
+        const int j = (it * THREADS + static_cast<int>(threadIdx.x)) * 4;
+        v[it].x += (y[it].x * post_scale) * wp[it].x;
+        v[it].y += (y[it].y * post_scale) * wp[it].y;
+        v[it].z += (y[it].z * post_scale) * wp[it].z;
+        v[it].w += (y[it].w * post_scale) * wp[it].w;
+        if (j < hidden) {
+            if (write_back) store4(res + j, v[it]);
+            sum_sq += v[it].x * v[it].x + v[it].y * v[it].y + v[it].z * v[it].z + v[it].w * v[it].w;
+        }
+    }
+    const float scale = 1.0f / sqrtf(block_sum(sum_sq, scratch) / static_cast<float>(hidden) + eps);
+    T* dst = out + static_cast<int64_t>(r) * hidden;
+#pragma unroll
+    for (int it = 0; it < ITERS; ++it) {
+        const int j = (it * THREADS + static_cast<int>(threadIdx.x)) * 4;
+        if (j < hidden)
+            store4(dst + j, float4{(v[it].x * scale) * w[it].x, (v[it].y * scale) * w[it].y, (v[it].z * scale) * w[it].z,
+                                   (v[it].w * scale) * w[it].w});
+    }
+}
+
 // One wave per (token, head): o [tokens][heads * width] float32 is normalised over the `width` values of
 // the head (plain weight [width], shared by the heads) and multiplied by act(gate) of the same place;
 // gate [tokens][gate_stride] of T (the columns of the head start at h * width).
@@ -98,6 +177,31 @@ extern "C" int fsie_sandwich_norm(float* residual, const void* delta, const floa
     FSIE_REQUIRE(!(write_back && rows), "sandwich_norm: chosen rows are read, not written back");
     if (n_rows == 0) return 0;
     const int64_t part_stride = static_cast<int64_t>(total_rows) * hidden;
+    const bool aligned = hidden % 4 == 0 && reinterpret_cast<uintptr_t>(residual) % 16 == 0 &&
+                         reinterpret_cast<uintptr_t>(delta) % 16 == 0 && reinterpret_cast<uintptr_t>(post_weight) % 16 == 0 &&
+                         reinterpret_cast<uintptr_t>(weight) % 16 == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0;
+    if (aligned && hidden <= 8192) {
+#define FSIE_SANDWICH(T, ITERS, THREADS)                                                                             \
+    sandwich_norm_vec_kernel<T, ITERS, THREADS><<<n_rows, THREADS, 0, stream>>>(                                     \
+        residual, static_cast<const T*>(delta), post_weight, post_eps, weight, eps, static_cast<T*>(out), rows, hidden, \
+        write_back, n_parts, part_stride)
+#define FSIE_SANDWICH_BY_SIZE(T)                                                      \
+    if (n_rows <= 128 && hidden > 1024) {  /* few rows: more waves a row */           \
+        if (hidden <= 4096) FSIE_SANDWICH(T, 1, 1024); else FSIE_SANDWICH(T, 2, 1024); \
+    } else if (hidden <= 1024) FSIE_SANDWICH(T, 1, 256);                              \
+    else if (hidden <= 2048) FSIE_SANDWICH(T, 2, 256);                                \
+    else if (hidden <= 4096) FSIE_SANDWICH(T, 4, 256);                                \
+    else FSIE_SANDWICH(T, 8, 256)
+        if (dtype == FSIE_F32) {
+            FSIE_SANDWICH_BY_SIZE(float);
+        } else {
+            FSIE_SANDWICH_BY_SIZE(bf16_t);
+        }
+#undef FSIE_SANDWICH_BY_SIZE
+#undef FSIE_SANDWICH
+        FSIE_CHECK_LAUNCH("sandwich_norm");
+        return 0;
+    }
     const size_t lds = sizeof(float) * hidden;
     if (dtype == FSIE_F32) {
         sandwich_norm_kernel<float><<<n_rows, kThreads, lds, stream>>>(residual, static_cast<const float*>(delta), post_weight,
