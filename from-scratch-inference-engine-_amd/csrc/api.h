@@ -63,16 +63,18 @@ int fsie_gated_act(const void* x, void* out, int n_tokens, int inter, int dtype,
 int fsie_sandwich_norm(float* residual, const void* delta, const float* post_weight, float post_eps, const float* weight,
                        float eps, void* out, const int32_t* rows, int n_rows, int hidden, int dtype, int write_back,
                        int n_parts, int total_rows, hipStream_t stream);
-// out[t][h][:] = rmsnorm(o[t][h][:]; weight, eps) * act(gate[t][h][:]), o float32, a head `width` values wide
-int fsie_gated_headnorm(const float* o, const void* gate, int64_t gate_stride, const float* weight, void* out, int n_tokens,
-                        int heads, int width, float eps, int act, int dtype, hipStream_t stream);
+// out[t][h][:] = rmsnorm(o[t][h][:]; weight, eps) * act(gate[t][h][:]), a head `width` values wide; o float32, the sum
+// in order of n_planes arrays [n_tokens][heads * width] that lie one after the other
+int fsie_gated_headnorm(const float* o, int n_planes, const void* gate, int64_t gate_stride, const float* weight, void* out,
+                        int n_tokens, int heads, int width, float eps, int act, int dtype, hipStream_t stream);
 // x <- cap * tanh(x / cap) in place
 int fsie_softcap(float* x, int64_t n, float cap, hipStream_t stream);
 
 // Gated linear attention over the tokens of a step, from and to the per-request state (linear_attention.hip).
+int fsie_gla_scan_shape(int heads, int dim, int vdim, int* prep_floats_per_token, int* out_planes);
 int fsie_gla_scan(const void* proj, int64_t proj_stride, int q_off, int k_off, int v_off, const float* z, float* state,
-                  const int32_t* q_starts, const int32_t* seq_slots, int n_seqs, float* out, int heads, int dim, int vdim,
-                  float q_scale, float inv_tau, int n_slots, int dtype, hipStream_t stream);
+                  const int32_t* q_starts, const int32_t* seq_slots, int n_seqs, int n_tokens, float* prep, float* out,
+                  int heads, int dim, int vdim, float q_scale, float inv_tau, int n_slots, int dtype, hipStream_t stream);
 
 // Attention through a latent (latent_attention.hip): the norms of the latents, the gates and the cache row of
 // every token; the rotation of pairs of neighbours; a product with a matrix of its own for every head.

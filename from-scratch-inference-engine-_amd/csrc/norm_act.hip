@@ -138,7 +138,7 @@ template <typename T>
 __global__ __launch_bounds__(kThreads) void gated_headnorm_kernel(const float* __restrict__ o, const T* __restrict__ gate,
                                                                   int64_t gate_stride, const float* __restrict__ weight,
                                                                   T* __restrict__ out, int64_t n_runs, int heads, int width,
-                                                                  float eps, int act) {
+                                                                  float eps, int act, int n_planes, int64_t plane) {
     const int lane = threadIdx.x & (FSIE_WAVE - 1);
     const int64_t run = static_cast<int64_t>(blockIdx.x) * (kThreads / FSIE_WAVE) + threadIdx.x / FSIE_WAVE;
     if (run >= n_runs) return;
@@ -147,12 +147,21 @@ __global__ __launch_bounds__(kThreads) void gated_headnorm_kernel(const float* _
     const float* src = o + (t * heads + h) * width;
     const T* g = gate + t * gate_stride + static_cast<int64_t>(h) * width;
     T* dst = out + (t * heads + h) * width;
+    // o comes as n_planes arrays a `plane` apart, added in order (the shares of a state kernel's row splits)
+    auto value = [&](int i) {
+        float x = src[i];
+        for (int p = 1; p < n_planes; ++p) x += src[p * plane + i];
+        return x;
+    };
     float sum = 0.f;
-    for (int i = lane; i < width; i += FSIE_WAVE) sum += src[i] * src[i];
+    for (int i = lane; i < width; i += FSIE_WAVE) {
+        const float x = value(i);
+        sum += x * x;
+    }
     sum = wave_sum(sum);
     const float scale = 1.0f / sqrtf(sum / static_cast<float>(width) + eps);
     for (int i = lane; i < width; i += FSIE_WAVE)
-        dst[i] = from_float<T>(((src[i] * scale) * weight[i]) * gate_act(to_float(g[i]), act));
+        dst[i] = from_float<T>(((value(i) * scale) * weight[i]) * gate_act(to_float(g[i]), act));
 }
 
 __global__ void softcap_kernel(float* __restrict__ x, int64_t n, float cap, float inv_cap) {
@@ -216,8 +225,11 @@ extern "C" int fsie_sandwich_norm(float* residual, const void* delta, const floa
     return 0;
 }
 
-extern "C" int fsie_gated_headnorm(const float* o, const void* gate, int64_t gate_stride, const float* weight, void* out,
-                                   int n_tokens, int heads, int width, float eps, int act, int dtype, hipStream_t stream) {
+extern "C" int fsie_gated_headnorm(const float* o, int n_planes, const void* gate, int64_t gate_stride, const float* weight,
+                                   void* out, int n_tokens, int heads, int width, float eps, int act, int dtype,
+                                   hipStream_t stream) {
+    FSIE_REQUIRE(n_planes >= 1, "gated_headnorm: at least one plane of o");
+    const int64_t plane = static_cast<int64_t>(n_tokens) * heads * width;
     FSIE_REQUIRE(n_tokens >= 0 && heads > 0 && width > 0, "gated_headnorm: bad sizes T=%d heads=%d width=%d", n_tokens, heads,
                  width);
     FSIE_REQUIRE(dtype == FSIE_F32 || dtype == FSIE_BF16, "gated_headnorm: unknown dtype %d", dtype);
@@ -229,10 +241,10 @@ extern "C" int fsie_gated_headnorm(const float* o, const void* gate, int64_t gat
     const unsigned grid = static_cast<unsigned>(ceil_div64(runs, kThreads / FSIE_WAVE));
     if (dtype == FSIE_F32) {
         gated_headnorm_kernel<float><<<grid, kThreads, 0, stream>>>(o, static_cast<const float*>(gate), gate_stride, weight,
-                                                                  static_cast<float*>(out), runs, heads, width, eps, act);
+                                                                  static_cast<float*>(out), runs, heads, width, eps, act, n_planes, plane);
     } else {
         gated_headnorm_kernel<bf16_t><<<grid, kThreads, 0, stream>>>(o, static_cast<const bf16_t*>(gate), gate_stride, weight,
-                                                                   static_cast<bf16_t*>(out), runs, heads, width, eps, act);
+                                                                   static_cast<bf16_t*>(out), runs, heads, width, eps, act, n_planes, plane);
     }
     FSIE_CHECK_LAUNCH("gated_headnorm");
     return 0;

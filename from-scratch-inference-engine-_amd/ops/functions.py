@@ -2,6 +2,8 @@
 
 from __future__ import annotations
 
+import ctypes
+
 from typing import Optional
 
 import torch
@@ -751,18 +753,21 @@ def sandwich_norm(residual: torch.Tensor, delta: torch.Tensor, post_weight: torc
 def gated_headnorm(o: torch.Tensor, gate: torch.Tensor, weight: torch.Tensor, eps: float, heads: int,
                    act: str = "silu") -> torch.Tensor:
     """``rmsnorm(o[t, h]; weight, eps) * act(gate[t, h])`` for every token and head: ``o`` float32
-    [T, heads * width], ``weight`` float32 [width] (shared by the heads), ``gate`` [T, heads * width] in the
-    activations' type (it may be columns of wider rows); the result has the gate's type."""
-    _need(o, "gated_headnorm o", dtype=torch.float32, ndim=2)
+    [T, heads * width] (or [P, T, heads * width]: planes that are added in order first), ``weight`` float32
+    [width] (shared by the heads), ``gate`` [T, heads * width] in the activations' type (it may be columns of
+    wider rows); the result has the gate's type."""
+    if o.dim() == 2:
+        o = o.unsqueeze(0)
+    _need(o, "gated_headnorm o", dtype=torch.float32, ndim=3)
     _need(weight, "gated_headnorm weight", dtype=torch.float32, ndim=1)
-    t, total = o.shape
+    planes, t, total = o.shape
     width = weight.shape[0]
     if total != heads * width:
         raise KernelError(f"gated_headnorm: rows of {total} values are not {heads} heads of {width}")
     if not gate.is_cuda or gate.dim() != 2 or gate.stride(1) != 1 or tuple(gate.shape) != (t, total):
         raise KernelError("gated_headnorm gate: must be [T, heads * width] on the GPU with contiguous rows")
     out = torch.empty((t, total), dtype=gate.dtype, device=o.device)
-    check(load().fsie_gated_headnorm(o.data_ptr(), gate.data_ptr(), gate.stride(0), weight.data_ptr(), out.data_ptr(), t,
+    check(load().fsie_gated_headnorm(o.data_ptr(), planes, gate.data_ptr(), gate.stride(0), weight.data_ptr(), out.data_ptr(), t,
                                      heads, width, float(eps), gate_act_code(act), dtype_code(gate.dtype), _stream()))
     return out
 
@@ -783,7 +788,9 @@ def gla_scan(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, z: torch.Te
     """S <- diag(sigmoid(z_t)^inv_tau) S + k_t v_t^T, o_t = S^T (q_scale q_t) over the tokens of every
     request of the step, from and to ``state`` float32 [slots, heads, dim, vdim].  ``proj`` [T, W] holds the
     q, k (heads x dim) and v (heads x vdim) columns from ``q_off``, ``k_off``, ``v_off``; ``z`` float32
-    [T, heads * dim]; ``q_starts`` int32 [n + 1], ``seq_slots`` int32 [n].  Returns o float32 [T, heads * vdim]."""
+    [T, heads * dim]; ``q_starts`` int32 [n + 1], ``seq_slots`` int32 [n].  Returns o float32 [P, T, heads * vdim]:
+    the shares of the P groups of key channels that the kernel deals a head's state to (P follows from the
+    sizes alone); their sum in order is o, and ``gated_headnorm`` takes them as they are."""
     _need(proj, "gla proj", ndim=2)
     t, w = proj.shape
     _need(z, "gla z", dtype=torch.float32, shape=(t, heads * dim))
@@ -795,10 +802,13 @@ def gla_scan(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, z: torch.Te
     n = seq_slots.shape[0]
     if q_starts.shape[0] != n + 1:
         raise KernelError("gla: q_starts must have one entry more than seq_slots")
-    out = torch.empty((t, heads * vdim), dtype=torch.float32, device=proj.device)
+    per_token, planes = ctypes.c_int(0), ctypes.c_int(0)
+    check(load().fsie_gla_scan_shape(heads, dim, vdim, ctypes.byref(per_token), ctypes.byref(planes)))
+    prep = torch.empty((t * per_token.value,), dtype=torch.float32, device=proj.device)
+    out = torch.empty((planes.value, t, heads * vdim), dtype=torch.float32, device=proj.device)
     check(load().fsie_gla_scan(proj.data_ptr(), w, q_off, k_off, v_off, z.data_ptr(), state.data_ptr(), q_starts.data_ptr(),
-                               seq_slots.data_ptr(), n, out.data_ptr(), heads, dim, vdim, float(q_scale), float(inv_tau),
-                               state.shape[0], dtype_code(proj.dtype), _stream()))
+                               seq_slots.data_ptr(), n, t, prep.data_ptr(), out.data_ptr(), heads, dim, vdim, float(q_scale),
+                               float(inv_tau), state.shape[0], dtype_code(proj.dtype), _stream()))
     return out
 
 

@@ -102,6 +102,9 @@ def test_softcap_and_gated_headnorm(ops):
         ref = plain.norm_plain_weight(o.double().reshape(t, heads, width), w.double(), 1e-5).reshape(t, -1) * g * torch.sigmoid(g)
         got = ops.gated_headnorm(o.cuda(), wide.cuda()[:, 11:], w.cuda(), 1e-5, heads)
         assert got.dtype == dtype and rel(got.float().cpu(), ref) <= tol(dtype, bf16=2.0 ** -7)
+        shares = torch.stack([0.5 * o, 0.25 * o, 0.25 * o]).cuda()  # o as three planes that are added first
+        got = ops.gated_headnorm(shares, wide.cuda()[:, 11:], w.cuda(), 1e-5, heads)
+        assert rel(got.float().cpu(), ref) <= tol(dtype, bf16=2.0 ** -7)
 
 
 def oracle_gla_states(q, k, v, z, tau, state):
@@ -137,7 +140,8 @@ def test_gla_scan_over_portions_and_slots(ops, dtype, heads, dim, vdim):
         z = torch.cat([data[r][1][lo:hi] for r, lo, hi in rows]).cuda()
         starts = np.cumsum([0] + [hi - lo for _, lo, hi in rows]).astype(np.int32)
         o = ops.gla_scan(proj, 5, 5 + kw, 5 + 2 * kw, z, state, torch.from_numpy(starts).cuda(),
-                         torch.tensor([slots[r] for r in order], dtype=torch.int32).cuda(), heads, dim, vdim, scale, 1 / tau).cpu()
+                         torch.tensor([slots[r] for r in order], dtype=torch.int32).cuda(), heads, dim, vdim, scale, 1 / tau)
+        o = o.sum(0).cpu()  # the shares of the groups of key channels
         for i, (r, lo, hi) in enumerate(rows):
             got[r].append(o[starts[i]:starts[i + 1]])
             fed[r] = hi
