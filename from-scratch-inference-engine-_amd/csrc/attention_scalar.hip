@@ -1,6 +1,7 @@
 // Causal grouped-query attention over the pages of the cache: float32 arithmetic throughout
 // (products, softmax, sums), for float32 or bfloat16 storage.  It is the attention of the 32-bit
-// path and takes any head size up to 256.
+// path and takes any head size up to 512 (beyond 256 in an instantiation with twice the accumulators
+// and more shared memory than a launch gets by default).
 //
 // The host cuts the step into work items (api.h: FSIE_ATTN_ITEM_*): a tile of up to 16/gh query
 // tokens of one request, a range of keys, and where the result goes: the output (normalised), or a
@@ -19,7 +20,8 @@ namespace {
 
 constexpr int kRows = 16;      // query rows per block
 constexpr int kKeys = 32;      // keys per tile
-constexpr int kMaxChunks = 8;  // head_dim <= 32 * 8
+constexpr int kMaxChunks = 8;       // head_dim <= 32 * 8: the usual instantiation
+constexpr int kMaxChunksWide = 16;  // head_dim <= 32 * 16
 
 __device__ __forceinline__ float half_wave_max(float v) {
 #pragma unroll
@@ -46,7 +48,7 @@ __device__ __forceinline__ void load4(const bf16_t* p, float (&f)[4]) {
 // VEC: the head size and the page size are multiples of 4 and the pools are aligned for load4, so a
 // thread copies four values of a key (along the head) or of a dimension (four consecutive slots of a
 // page; only for items whose first key is a multiple of 4, else element by element) with one load.
-template <typename T, bool VEC>
+template <typename T, bool VEC, int MAXC>
 __global__ __launch_bounds__(256) void attention_scalar_kernel(
     const T* __restrict__ q, int64_t q_stride, const T* __restrict__ k_pool, const T* __restrict__ v_pool,
     const int32_t* __restrict__ block_tables, int max_pages, const int32_t* __restrict__ items,
@@ -92,13 +94,13 @@ __global__ __launch_bounds__(256) void attention_scalar_kernel(
         qs[e] = v;
     }
 
-    float m_run[2], l_run[2], acc[2][kMaxChunks];
+    float m_run[2], l_run[2], acc[2][MAXC];
 #pragma unroll
     for (int p = 0; p < 2; ++p) {
         m_run[p] = -INFINITY;
         l_run[p] = 0.f;
 #pragma unroll
-        for (int i = 0; i < kMaxChunks; ++i) acc[p][i] = 0.f;
+        for (int i = 0; i < MAXC; ++i) acc[p][i] = 0.f;
     }
     const int n_chunks = (hd + 31) / 32;
     const int32_t* table = block_tables + static_cast<int64_t>(seq) * max_pages;
@@ -195,7 +197,7 @@ __global__ __launch_bounds__(256) void attention_scalar_kernel(
             const int r = wave * 4 + p * 2 + sub;
             const float* pr = ps + r * kKeys;
 #pragma unroll
-            for (int i = 0; i < kMaxChunks; ++i) {
+            for (int i = 0; i < MAXC; ++i) {
                 if (i < n_chunks) {
                     const int d = lane32 + 32 * i;
                     float a = acc[p][i] * corr[p];
@@ -220,14 +222,14 @@ __global__ __launch_bounds__(256) void attention_scalar_kernel(
             const float inv = denom > 0.f ? 1.0f / denom : 0.f;
             T* o = out + (static_cast<int64_t>(q_row0 + tq) * n_heads + hq) * hd;
 #pragma unroll
-            for (int i = 0; i < kMaxChunks; ++i) {
+            for (int i = 0; i < MAXC; ++i) {
                 const int d = lane32 + 32 * i;
                 if (i < n_chunks && d < hd) o[d] = from_float<T>(acc[p][i] * inv);
             }
         } else {
             float* rec = partials + (static_cast<int64_t>(partial_base + tq) * n_heads + hq) * (hd + 2);
 #pragma unroll
-            for (int i = 0; i < kMaxChunks; ++i) {
+            for (int i = 0; i < MAXC; ++i) {
                 const int d = lane32 + 32 * i;
                 if (i < n_chunks && d < hd) rec[d] = acc[p][i];
             }
@@ -375,7 +377,8 @@ void launch_merge(const float* partials, const int32_t* merges, int n_merges, T*
     const dim3 grid(n_merges, n_heads);
     if (hd <= 64) attention_merge_kernel<T, 1><<<grid, 256, 0, stream>>>(partials, merges, out, n_heads, hd, sinks);
     else if (hd <= 128) attention_merge_kernel<T, 2><<<grid, 256, 0, stream>>>(partials, merges, out, n_heads, hd, sinks);
-    else attention_merge_kernel<T, 4><<<grid, 256, 0, stream>>>(partials, merges, out, n_heads, hd, sinks);
+    else if (hd <= 256) attention_merge_kernel<T, 4><<<grid, 256, 0, stream>>>(partials, merges, out, n_heads, hd, sinks);
+    else attention_merge_kernel<T, 8><<<grid, 256, 0, stream>>>(partials, merges, out, n_heads, hd, sinks);
 }
 
 }  // namespace
@@ -387,8 +390,8 @@ extern "C" int fsie_attention_scalar(const void* q, int64_t q_stride, const void
                                      const float* sinks, hipStream_t stream) {
     FSIE_REQUIRE(n_items >= 0 && n_heads > 0 && n_kv > 0 && n_heads % n_kv == 0,
                  "attention: heads %d must be a positive multiple of kv heads %d", n_heads, n_kv);
-    FSIE_REQUIRE(head_dim > 0 && head_dim <= 32 * kMaxChunks, "attention: head_dim %d must be in 1..%d",
-                 head_dim, 32 * kMaxChunks);
+    FSIE_REQUIRE(head_dim > 0 && head_dim <= 32 * kMaxChunksWide, "attention: head_dim %d must be in 1..%d",
+                 head_dim, 32 * kMaxChunksWide);
     FSIE_REQUIRE(page_size > 0 && max_pages > 0, "attention: bad page geometry");
     FSIE_REQUIRE(dtype == FSIE_F32 || dtype == FSIE_BF16, "attention: unknown dtype %d", dtype);
     if (n_items == 0) return 0;
@@ -399,19 +402,36 @@ extern "C" int fsie_attention_scalar(const void* q, int64_t q_stride, const void
     const size_t lds = sizeof(float) * (static_cast<size_t>(kRows) * head_dim + kKeys * (head_dim + 1) + kRows * kKeys);
     const bool vec = head_dim % 4 == 0 && page_size % 4 == 0 && reinterpret_cast<uintptr_t>(k_pool) % 16 == 0 &&
                      reinterpret_cast<uintptr_t>(v_pool) % 16 == 0;
-    if (dtype == FSIE_F32) {
-        auto kernel = vec ? attention_scalar_kernel<float, true> : attention_scalar_kernel<float, false>;
-        kernel<<<grid, 256, lds, stream>>>(
-            static_cast<const float*>(q), q_stride, static_cast<const float*>(k_pool), static_cast<const float*>(v_pool),
-            block_tables, max_pages, items, static_cast<float*>(out), partials, n_heads, n_kv, head_dim, page_size,
-            window, scale, gh, head_chunks, sinks);
-    } else {
-        auto kernel = vec ? attention_scalar_kernel<bf16_t, true> : attention_scalar_kernel<bf16_t, false>;
-        kernel<<<grid, 256, lds, stream>>>(
-            static_cast<const bf16_t*>(q), q_stride, static_cast<const bf16_t*>(k_pool),
-            static_cast<const bf16_t*>(v_pool), block_tables, max_pages, items, static_cast<bf16_t*>(out), partials,
-            n_heads, n_kv, head_dim, page_size, window, scale, gh, head_chunks, sinks);
+    const bool wide = head_dim > 32 * kMaxChunks;
+#define FSIE_SCALAR_ATTENTION(T, VEC, MAXC)                                                                          \
+    do {                                                                                                             \
+        auto kernel = attention_scalar_kernel<T, VEC, MAXC>;                                                         \
+        if (lds > 48 * 1024) {  /* more shared memory than a launch gets unasked */                                  \
+            const hipError_t allowed = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),                    \
+                                                           hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)); \
+            FSIE_REQUIRE(allowed == hipSuccess, "attention: %zu bytes of shared memory for head_dim %d: %s", lds, head_dim, \
+                         hipGetErrorString(allowed));                                                                \
+        }                                                                                                            \
+        kernel<<<grid, 256, lds, stream>>>(static_cast<const T*>(q), q_stride, static_cast<const T*>(k_pool),        \
+                                           static_cast<const T*>(v_pool), block_tables, max_pages, items,            \
+                                           static_cast<T*>(out), partials, n_heads, n_kv, head_dim, page_size, window, \
+                                           scale, gh, head_chunks, sinks);                                           \
+    } while (0)
+#define FSIE_SCALAR_ATTENTION_OF(T)                                          \
+    if (wide) {                                                              \
+        if (vec) FSIE_SCALAR_ATTENTION(T, true, kMaxChunksWide);             \
+        else FSIE_SCALAR_ATTENTION(T, false, kMaxChunksWide);                \
+    } else {                                                                 \
+        if (vec) FSIE_SCALAR_ATTENTION(T, true, kMaxChunks);                 \
+        else FSIE_SCALAR_ATTENTION(T, false, kMaxChunks);                    \
     }
+    if (dtype == FSIE_F32) {
+        FSIE_SCALAR_ATTENTION_OF(float)
+    } else {
+        FSIE_SCALAR_ATTENTION_OF(bf16_t)
+    }
+#undef FSIE_SCALAR_ATTENTION_OF
+#undef FSIE_SCALAR_ATTENTION
     FSIE_CHECK_LAUNCH("attention_scalar");
     return 0;
 }
@@ -419,7 +439,7 @@ extern "C" int fsie_attention_scalar(const void* q, int64_t q_stride, const void
 extern "C" int fsie_attention_merge(const float* partials, const int32_t* merges, int n_merges, void* out,
                                     int n_heads, int head_dim, int dtype, const float* sinks, hipStream_t stream) {
     FSIE_REQUIRE(n_merges >= 0 && n_heads > 0 && head_dim > 0, "attention_merge: bad sizes");
-    FSIE_REQUIRE(head_dim <= 256, "attention_merge: head_dim %d is larger than 256", head_dim);
+    FSIE_REQUIRE(head_dim <= 512, "attention_merge: head_dim %d is larger than 512", head_dim);
     FSIE_REQUIRE(dtype == FSIE_F32 || dtype == FSIE_BF16, "attention_merge: unknown dtype %d", dtype);
     if (n_merges == 0) return 0;
     if (dtype == FSIE_F32) launch_merge(partials, merges, n_merges, static_cast<float*>(out), n_heads, head_dim, sinks, stream);

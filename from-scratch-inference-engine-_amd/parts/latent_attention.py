@@ -12,7 +12,7 @@ from .attention import AttentionPlanner, paged_attention
 from .base import Mixer, ParamDecl, Part, PositionEncoding, register_part
 from .linear import Linear
 
-MAX_WIDTH = 256  # the widest cache row that the attention kernels take
+MAX_WIDTH = 512  # the widest cache row that an attention kernel takes (the matrix-core kernels: 256)
 
 
 @register_part("mixer", "latent_attention")
@@ -25,7 +25,8 @@ class LatentAttention(Mixer):
     sigmoid(W_g x)_h (``gate=True``), and W_o over the heads.
 
     Only c and the shared part are cached: one row of ``width`` values a token (their sum rounded up to 16,
-    zeros at the end) in a paged cache of a single kv head.  Attention runs over those rows as they are,
+    zeros at the end; up to 256 values the matrix-core kernels serve bfloat16, wider rows up to 512 go to the
+    float32-arithmetic kernel in both precisions) in a paged cache of a single kv head.  Attention runs over those rows as they are,
     with the engine's kernels for grouped queries (every head reads the same keys): head h's query becomes
     [W_uk,h^T q_h | turned part], the values are the rows themselves, and W_uv,h is applied to the result.
     ``own_latent=False``: the layer has no W_dkv and reads the cache of the layer that the model's schedule
