@@ -71,10 +71,12 @@ int fsie_gated_headnorm(const float* o, int n_planes, const void* gate, int64_t 
 int fsie_softcap(float* x, int64_t n, float cap, hipStream_t stream);
 
 // Gated linear attention over the tokens of a step, from and to the per-request state (linear_attention.hip).
-int fsie_gla_scan_shape(int heads, int dim, int vdim, int* prep_floats_per_token, int* out_planes);
+int fsie_gla_scan_shape(int heads, int dim, int vdim, int* prep_floats_per_token, int* out_planes, int* chunk_tokens,
+                        int* chunk_min, int64_t* chunk_floats);
 int fsie_gla_scan(const void* proj, int64_t proj_stride, int q_off, int k_off, int v_off, const float* z, float* state,
                   const int32_t* q_starts, const int32_t* seq_slots, int n_seqs, int n_tokens, float* prep, float* out,
-                  int heads, int dim, int vdim, float q_scale, float inv_tau, int n_slots, int dtype, hipStream_t stream);
+                  float* chunk_work, int max_chunks, int heads, int dim, int vdim, float q_scale, float inv_tau,
+                  int n_slots, int dtype, hipStream_t stream);
 
 // Attention through a latent (latent_attention.hip): the norms of the latents, the gates and the cache row of
 // every token; the rotation of pairs of neighbours; a product with a matrix of its own for every head.

@@ -13,6 +13,19 @@
 // the same in all its lanes: a first kernel lays these out in float32 ([token][head][padded channel], the
 // padding with decay 1 and k = q = 0), and the walk reads them with addresses that are uniform over the
 // wave, which the compiler turns into scalar loads: no lane-wide traffic for them at all.
+//
+// A portion of kGlaChunkMin tokens or more does not walk token by token.  It is cut into chunks of sixteen
+// tokens (counted from the portion's first token), and with B_t the sum of log alpha over the chunk's tokens
+// up to and including t, per channel,
+//   o_t   = (q_t * exp(B_t))^T S_in + sum_{j <= t} A[t][j] v_j,   A[t][j] = sum_c q_t[c] k_j[c] exp(B_t[c] - B_j[c]),
+//   S_out = diag(exp(B_last)) S_in + sum_j (k_j * exp(B_last - B_j)) v_j^T,
+// which is the same recurrence with its sums taken in another order: every exponent is a sum of logarithms of
+// decays, none is positive, nothing can overflow whatever the decays are.  A first kernel computes the scaled
+// q and k, the chunk's decay and A for every chunk and head at once (float32 on the vector units); the walk
+// over chunks then is three small matrix products a chunk on the float32 matrix instruction
+// (v_mfma_f32_16x16x4_f32, no rounding of operands), one wave per sixteen key channels and sixteen value
+// columns with its tile of S in an accumulator; the waves of a head's columns meet once a chunk to add their
+// shares of o.
 #include "common.h"
 #include "api.h"
 
@@ -24,6 +37,11 @@ constexpr int kGlaWaves = 16;
 constexpr int kGlaThreads = 64 * kGlaWaves;
 constexpr int kGlaCols = 64;
 constexpr int kGlaTokens = 8;  // tokens whose shares of o are added up at once
+constexpr int kGlaChunk = 16;     // tokens of a chunk: one tile of the matrix instruction
+constexpr int kGlaChunkMin = 16;  // portions of at least this many tokens go chunk by chunk
+constexpr int kGlaChunkThreads = 256;
+
+typedef float floatx4 __attribute__((ext_vector_type(4)));
 
 // log(sigmoid(z)) without overflow: min(z, 0) - log(1 + exp(-|z|))
 __device__ __forceinline__ float log_sigmoid(float z) { return fminf(z, 0.f) - log1pf(expf(-fabsf(z))); }
@@ -63,7 +81,8 @@ template <typename T, int ROWS>
 __global__ __launch_bounds__(kGlaThreads) void gla_scan_kernel(
     const T* __restrict__ proj, int64_t proj_stride, int v_off, const float* __restrict__ prep, int64_t prep_plane,
     float* __restrict__ state, const int32_t* __restrict__ q_starts, const int32_t* __restrict__ seq_slots,
-    float* __restrict__ out, int64_t out_plane, int heads, int dim, int vdim, int dp, int row_splits, int n_slots) {
+    float* __restrict__ out, int64_t out_plane, int heads, int dim, int vdim, int dp, int row_splits, int n_slots,
+    int skip_from) {
     constexpr int TT = kGlaTokens;
     __shared__ float part[kGlaWaves][TT][kGlaCols];
     const int seq = blockIdx.x, h = blockIdx.y;
@@ -74,6 +93,7 @@ __global__ __launch_bounds__(kGlaThreads) void gla_scan_kernel(
     const int lo = q_starts[seq], hi = q_starts[seq + 1];
     const int slot = seq_slots[seq];
     if (hi <= lo || slot < 0 || slot >= n_slots) return;  // the same for the whole workgroup
+    if (hi - lo >= skip_from) return;                     // the chunk kernels' portion
     const bool col_ok = col < vdim;
     const int row0 = (split * kGlaWaves + wave) * ROWS;  // this wave's first key channel
 
@@ -128,6 +148,201 @@ __global__ __launch_bounds__(kGlaThreads) void gla_scan_kernel(
     }
 }
 
+// The chunks of a step are numbered request by request, in the order of the requests; a request whose portion
+// is shorter than kGlaChunkMin, or that has no slot, has none.  (A handful of scalar loads per workgroup.)
+__device__ __forceinline__ int gla_chunks_of(const int32_t* q_starts, const int32_t* seq_slots, int s, int n_slots) {
+    const int len = q_starts[s + 1] - q_starts[s];
+    const int slot = seq_slots[s];
+    return (len >= kGlaChunkMin && slot >= 0 && slot < n_slots) ? (len + kGlaChunk - 1) / kGlaChunk : 0;
+}
+
+// Work array of one chunk and head: qd [16][dp] (q * exp(B_t)), kdT [dp][16] (k * exp(B_last - B_t), channel
+// major), g [dp] (exp(B_last)), A [16][16] (zero above the diagonal).  Tokens past the portion's end and
+// channels past dim count as decay 1 with q = k = 0.
+__host__ __device__ inline int64_t gla_chunk_floats(int dp) { return static_cast<int64_t>(2 * kGlaChunk + 1) * dp + kGlaChunk * kGlaChunk; }
+
+// grid = (upper bound of the step's chunks, heads).
+template <typename T>
+__global__ __launch_bounds__(kGlaChunkThreads) void gla_chunk_prep_kernel(
+    const T* __restrict__ proj, int64_t proj_stride, int q_off, int k_off, const float* __restrict__ z,
+    float* __restrict__ work, const int32_t* __restrict__ q_starts, const int32_t* __restrict__ seq_slots, int n_seqs,
+    int heads, int dim, int dp, float q_scale, float inv_tau, int n_slots) {
+    extern __shared__ float lds[];  // [3][16][dp + 1]: q, k, B
+    const int ld = dp + 1;
+    float* qs = lds;
+    float* ks = qs + kGlaChunk * ld;
+    float* bs = ks + kGlaChunk * ld;
+    const int h = blockIdx.y, tid = threadIdx.x;
+    int first = 0, seq = -1;
+    for (int s = 0; s < n_seqs; ++s) {
+        const int n = gla_chunks_of(q_starts, seq_slots, s, n_slots);
+        if (static_cast<int>(blockIdx.x) < first + n) { seq = s; break; }
+        first += n;
+    }
+    if (seq < 0) return;  // the same for the whole workgroup
+    const int t0 = q_starts[seq] + (static_cast<int>(blockIdx.x) - first) * kGlaChunk;
+    const int nt = min(kGlaChunk, q_starts[seq + 1] - t0);
+    float* w = work + (static_cast<int64_t>(blockIdx.x) * heads + h) * gla_chunk_floats(dp);
+    float* qd = w;
+    float* kdT = qd + kGlaChunk * dp;
+    float* g = kdT + kGlaChunk * dp;
+    float* A = g + dp;
+
+    for (int c = tid; c < dp; c += kGlaChunkThreads) {
+        float q[kGlaChunk], k[kGlaChunk], b[kGlaChunk];
+        float sum = 0.f;
+#pragma unroll
+        for (int t = 0; t < kGlaChunk; ++t) {
+            q[t] = 0.f;
+            k[t] = 0.f;
+            if (t < nt && c < dim) {
+                const T* row = proj + static_cast<int64_t>(t0 + t) * proj_stride + h * dim + c;
+                q[t] = to_float(row[q_off]) * q_scale;
+                k[t] = to_float(row[k_off]);
+                sum += inv_tau * log_sigmoid(z[(static_cast<int64_t>(t0 + t) * heads + h) * dim + c]);
+            }
+            b[t] = sum;
+            qs[t * ld + c] = q[t];
+            ks[t * ld + c] = k[t];
+            bs[t * ld + c] = sum;
+        }
+        floatx4 kd[kGlaChunk / 4];
+#pragma unroll
+        for (int t = 0; t < kGlaChunk; ++t) {
+            qd[t * dp + c] = q[t] * expf(b[t]);
+            kd[t / 4][t % 4] = k[t] * expf(sum - b[t]);
+        }
+#pragma unroll
+        for (int t4 = 0; t4 < kGlaChunk / 4; ++t4) *reinterpret_cast<floatx4*>(kdT + c * kGlaChunk + 4 * t4) = kd[t4];
+        g[c] = expf(sum);
+    }
+    __syncthreads();
+    for (int e = tid; e < kGlaChunk * kGlaChunk; e += kGlaChunkThreads) {
+        const int i = e / kGlaChunk, j = e % kGlaChunk;
+        float a = 0.f;
+        if (j <= i && i < nt) {
+            for (int c = 0; c < dim; ++c) a = fmaf(qs[i * ld + c] * ks[j * ld + c], expf(bs[i * ld + c] - bs[j * ld + c]), a);
+        }
+        A[e] = a;
+    }
+}
+
+// grid = (requests of the step, heads, tiles of sixteen value columns); a workgroup has a wave for every
+// sixteen key channels of the head (NW: their number, rounded up to a power of two), and wave w holds the tile S[16 w .. 16 w + 15][its columns] in an
+// accumulator: lane l has the channels 4 (l / 16) .. + 3 of it at the column l % 16.  That is also the layout of
+// the instruction's second operand over four steps, if step i takes the channels 4 g + i (g = 0..3) as its four
+// inner indices; a sum does not mind the order, so S is multiplied from the left as it lies.  The same
+// renumbering of the inner index (the tokens 4 g + m at step m) lets v, kdT and A be read in vectors of four.
+// A wave's chain per chunk is nine matrix instructions; the waves' shares of the chunk's o (and the four steps
+// of A v, dealt to the waves in turn) meet in shared memory once a chunk and are added in the order of the
+// waves.  The shares of o that the token-by-token kernel would leave in further planes of `out` are zero here.
+template <typename T, int NW>
+__global__ __launch_bounds__(64 * NW) void gla_chunk_scan_kernel(
+    const T* __restrict__ proj, int64_t proj_stride, int v_off, const float* __restrict__ work,
+    float* __restrict__ state, const int32_t* __restrict__ q_starts, const int32_t* __restrict__ seq_slots,
+    float* __restrict__ out, int64_t out_plane, int heads, int dim, int vdim, int dp, int planes, int n_slots) {
+    __shared__ float part[2][NW][4][64];
+    const int seq = blockIdx.x, h = blockIdx.y;
+    const int n_chunks = gla_chunks_of(q_starts, seq_slots, seq, n_slots);
+    if (n_chunks == 0) return;  // the same for the whole workgroup
+    int first = 0;
+    for (int s = 0; s < seq; ++s) first += gla_chunks_of(q_starts, seq_slots, s, n_slots);
+    const int lo = q_starts[seq], hi = q_starts[seq + 1], slot = seq_slots[seq];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int n = lane & 15, g4 = lane >> 4;
+    const int col = blockIdx.z * 16 + n;
+    const bool col_ok = col < vdim;
+    const int ch0 = wave * 16;  // this wave's first key channel
+
+    float* my_state = state + ((static_cast<int64_t>(slot) * heads + h) * dim) * vdim + col;
+    floatx4 S;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int row = ch0 + 4 * g4 + i;
+        S[i] = (col_ok && row < dim) ? my_state[static_cast<int64_t>(row) * vdim] : 0.f;
+    }
+    const int64_t per_chunk = gla_chunk_floats(dp) * heads;
+    const float* w = work + (static_cast<int64_t>(first) * heads + h) * gla_chunk_floats(dp);
+    const T* vp = proj + v_off + h * vdim + min(col, vdim - 1);  // (columns past the head's last: a number, unused)
+    const int64_t out_stride = static_cast<int64_t>(heads) * vdim;
+
+    // The operands of the next D - 1 chunks are on their way while a chunk is multiplied: a ring of D sets of
+    // registers, the walk unrolled D times so that every set has a fixed place.
+    constexpr int D = 4;
+    floatx4 q4[D], k4[D], g4v[D], a4[D];
+    float v[D][4];
+    auto fetch = [&](const int slot_, int ci) {
+        ci = min(ci, n_chunks - 1);  // past the end: the last chunk once more, never used
+        const float* wc = w + ci * per_chunk;
+        const int t0 = lo + ci * kGlaChunk;
+#pragma unroll
+        for (int m = 0; m < 4; ++m) {
+            const int t = min(t0 + 4 * g4 + m, hi - 1);
+            v[slot_][m] = to_float(vp[static_cast<int64_t>(t) * proj_stride]);
+        }
+        q4[slot_] = *reinterpret_cast<const floatx4*>(wc + n * dp + ch0 + 4 * g4);
+        k4[slot_] = *reinterpret_cast<const floatx4*>(wc + kGlaChunk * dp + (ch0 + n) * kGlaChunk + 4 * g4);
+        g4v[slot_] = *reinterpret_cast<const floatx4*>(wc + 2 * kGlaChunk * dp + ch0 + 4 * g4);
+        a4[slot_] = *reinterpret_cast<const floatx4*>(wc + (2 * kGlaChunk + 1) * dp + n * kGlaChunk + 4 * g4);
+    };
+#pragma unroll
+    for (int u = 0; u < D - 1; ++u) fetch(u, u);
+    for (int base = 0; base < n_chunks; base += D) {
+#pragma unroll
+        for (int u = 0; u < D; ++u) {
+            const int ci = base + u;
+            if (ci < n_chunks) {  // the same for the whole workgroup
+                fetch((u + D - 1) % D, ci + D - 1);
+                const int t0 = lo + ci * kGlaChunk;
+                // (a token past the portion's end has k = 0 and a zero row of A: whatever v was read for it
+                // is multiplied by zero, but it must be a number)
+                float cv[4];
+#pragma unroll
+                for (int m = 0; m < 4; ++m) cv[m] = (t0 + 4 * g4 + m < hi && col_ok) ? v[u][m] : 0.f;
+                floatx4 o[4];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    o[i] = __builtin_amdgcn_mfma_f32_16x16x4f32(q4[u][i], S[i], floatx4{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+                }
+#pragma unroll
+                for (int m = 0; m < 4; ++m) {
+                    if (m % NW == wave) o[m] = __builtin_amdgcn_mfma_f32_16x16x4f32(a4[u][m], cv[m], o[m], 0, 0, 0);
+                }
+                S *= g4v[u];
+#pragma unroll
+                for (int m = 0; m < 4; ++m) S = __builtin_amdgcn_mfma_f32_16x16x4f32(k4[u][m], cv[m], S, 0, 0, 0);
+                const floatx4 mine = (o[0] + o[1]) + (o[2] + o[3]);
+#pragma unroll
+                for (int i = 0; i < 4; ++i) part[ci & 1][wave][i][lane] = mine[i];
+                lds_barrier();
+                // (the barrier of the next chunk keeps its writers off this half until everyone has read it)
+#pragma unroll
+                for (int e0 = 0; e0 < 256; e0 += 64 * NW) {
+                    const int e = e0 + tid;
+                    if (e < 256) {
+                        const int i = e >> 6, l = e & 63;
+                        float sum = part[ci & 1][0][i][l];
+#pragma unroll
+                        for (int ww = 1; ww < NW; ++ww) sum += part[ci & 1][ww][i][l];
+                        const int t = t0 + 4 * (l >> 4) + i, cc = blockIdx.z * 16 + (l & 15);
+                        if (t < hi && cc < vdim) {
+                            float* dst = out + static_cast<int64_t>(t) * out_stride + h * vdim + cc;
+                            *dst = sum;
+                            for (int pl = 1; pl < planes; ++pl) dst[pl * out_plane] = 0.f;
+                        }
+                    }
+                }
+            }
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int row = ch0 + 4 * g4 + i;
+        if (col_ok && row < dim) my_state[static_cast<int64_t>(row) * vdim] = S[i];
+    }
+}
+
 // Key channels a wave holds and the splits of a head's channels over workgroups: as many splits (1, 2, 4)
 // as still leave a wave four channels, while the workgroups of one request number fewer than 128.  A
 // function of the layer's sizes alone, never of the step.
@@ -144,14 +359,20 @@ void gla_shape(int heads, int dim, int vdim, int* rows, int* splits) {
 
 }  // namespace
 
-// Sizes of the two work arrays of fsie_gla_scan for a layer of these sizes: floats of `prep` a token, and the
-// planes of `out` (row splits).
-extern "C" int fsie_gla_scan_shape(int heads, int dim, int vdim, int* prep_floats_per_token, int* out_planes) {
+// Sizes of the work arrays of fsie_gla_scan for a layer of these sizes: floats of `prep` a token, the planes
+// of `out` (row splits), and for the portions that go chunk by chunk the tokens of a chunk, the shortest such
+// portion and the floats of `chunk_work` a chunk.  A step of n_tokens tokens in n_seqs requests has at most
+// n_tokens / chunk_tokens + n_seqs chunks, and none if n_tokens < chunk_min.
+extern "C" int fsie_gla_scan_shape(int heads, int dim, int vdim, int* prep_floats_per_token, int* out_planes,
+                                   int* chunk_tokens, int* chunk_min, int64_t* chunk_floats) {
     FSIE_REQUIRE(heads > 0 && dim > 0 && dim <= 256 && vdim > 0, "gla_scan_shape: bad sizes");
     int rows, splits;
     gla_shape(heads, dim, vdim, &rows, &splits);
     *prep_floats_per_token = 3 * heads * kGlaWaves * splits * rows;
     *out_planes = splits;
+    *chunk_tokens = kGlaChunk;
+    *chunk_min = kGlaChunkMin;
+    *chunk_floats = gla_chunk_floats(kGlaWaves * splits * rows) * heads;
     return 0;
 }
 
@@ -161,11 +382,14 @@ extern "C" int fsie_gla_scan_shape(int heads, int dim, int vdim, int* prep_float
 // q_starts[s] .. q_starts[s + 1] and the slot seq_slots[s] (a slot outside the table: the request is
 // skipped).  q is multiplied by q_scale; alpha = sigmoid(z)^inv_tau.  prep: work array of n_tokens *
 // prep_floats_per_token floats; out: out_planes arrays [n_tokens][heads * vdim] float32 whose sum, in order,
-// is o (fsie_gla_scan_shape gives both numbers).
+// is o (fsie_gla_scan_shape gives both numbers).  chunk_work: room for max_chunks chunks, or null: with it, the
+// portions of at least chunk_min tokens go chunk by chunk (max_chunks must be the bound that fsie_gla_scan_shape
+// names, or more); without it every portion is walked token by token.  Which way a portion goes depends on
+// its own length alone, and the two ways differ by rounding only.
 extern "C" int fsie_gla_scan(const void* proj, int64_t proj_stride, int q_off, int k_off, int v_off, const float* z,
                              float* state, const int32_t* q_starts, const int32_t* seq_slots, int n_seqs, int n_tokens,
-                             float* prep, float* out, int heads, int dim, int vdim, float q_scale, float inv_tau,
-                             int n_slots, int dtype, hipStream_t stream) {
+                             float* prep, float* out, float* chunk_work, int max_chunks, int heads, int dim, int vdim,
+                             float q_scale, float inv_tau, int n_slots, int dtype, hipStream_t stream) {
     FSIE_REQUIRE(n_seqs >= 0 && n_tokens >= 0 && heads > 0 && dim > 0 && vdim > 0 && n_slots > 0, "gla_scan: bad sizes");
     FSIE_REQUIRE(dim <= 256, "gla_scan: %d key channels a head are more than the kernel takes (256)", dim);
     FSIE_REQUIRE(dtype == FSIE_F32 || dtype == FSIE_BF16, "gla_scan: unknown dtype %d", dtype);
@@ -178,15 +402,31 @@ extern "C" int fsie_gla_scan(const void* proj, int64_t proj_stride, int q_off, i
     gla_shape(heads, dim, vdim, &rows, &splits);
     const int dp = kGlaWaves * splits * rows;
     const int col_blocks = (vdim + kGlaCols - 1) / kGlaCols;
-    FSIE_REQUIRE(heads <= 65535 && col_blocks * splits <= 65535, "gla_scan: too many heads or columns");
+    FSIE_REQUIRE(heads <= 65535 && col_blocks * splits <= 65535 && (vdim + 15) / 16 <= 65535, "gla_scan: too many heads or columns");
     const int64_t plane = static_cast<int64_t>(n_tokens) * heads * dp;
     const int64_t out_plane = static_cast<int64_t>(n_tokens) * heads * vdim;
     const unsigned prep_grid = static_cast<unsigned>(ceil_div64(plane, 256));
     const dim3 grid(n_seqs, heads, col_blocks * splits);
+    const bool chunks = chunk_work != nullptr && n_tokens >= kGlaChunkMin;
+    if (chunks) {
+        FSIE_REQUIRE(max_chunks >= n_tokens / kGlaChunk + n_seqs, "gla_scan: room for %d chunks, the step may have %d",
+                     max_chunks, n_tokens / kGlaChunk + n_seqs);
+        FSIE_REQUIRE(max_chunks <= 0x7fffffff / kGlaChunk, "gla_scan: too many chunks");
+    }
+    const int skip_from = chunks ? kGlaChunkMin : 0x7fffffff;
+    const dim3 chunk_grid(chunks ? max_chunks : 1, heads);
+    const size_t chunk_lds = 3 * kGlaChunk * (dp + 1) * sizeof(float);
+    const dim3 scan_grid(n_seqs, heads, (vdim + 15) / 16);
+    int scan_waves = 1;  // a wave for every sixteen key channels, rounded up to a power of two: at most sixteen
+    while (scan_waves * 16 < dim) scan_waves *= 2;
+#define FSIE_GLA_CHUNKS(T, NW)                                                                                        \
+    gla_chunk_scan_kernel<T, NW><<<scan_grid, 64 * NW, 0, stream>>>(static_cast<const T*>(proj), proj_stride, v_off,    \
+                                                                    chunk_work, state, q_starts, seq_slots, out,        \
+                                                                    out_plane, heads, dim, vdim, dp, splits, n_slots)
 #define FSIE_GLA_LAUNCH(T, ROWS)                                                                                       \
     gla_scan_kernel<T, ROWS><<<grid, kGlaThreads, 0, stream>>>(static_cast<const T*>(proj), proj_stride, v_off, prep, plane, \
                                                                state, q_starts, seq_slots, out, out_plane, heads, dim, vdim, \
-                                                               dp, splits, n_slots)
+                                                               dp, splits, n_slots, skip_from)
 #define FSIE_GLA_BY_ROWS(T)                                                                                          \
     gla_prep_kernel<T><<<prep_grid, 256, 0, stream>>>(static_cast<const T*>(proj), proj_stride, q_off, k_off, z, prep, \
                                                       plane, heads, dim, dp, q_scale, inv_tau);                      \
@@ -194,7 +434,17 @@ extern "C" int fsie_gla_scan(const void* proj, int64_t proj_stride, int q_off, i
     else if (rows == 2) FSIE_GLA_LAUNCH(T, 2);                                                                       \
     else if (rows == 4) FSIE_GLA_LAUNCH(T, 4);                                                                       \
     else if (rows == 8) FSIE_GLA_LAUNCH(T, 8);                                                                       \
-    else FSIE_GLA_LAUNCH(T, 16)
+    else FSIE_GLA_LAUNCH(T, 16);                                                                                     \
+    if (chunks) {                                                                                                    \
+        gla_chunk_prep_kernel<T><<<chunk_grid, kGlaChunkThreads, chunk_lds, stream>>>(                                \
+            static_cast<const T*>(proj), proj_stride, q_off, k_off, z, chunk_work, q_starts, seq_slots, n_seqs, heads, dim, \
+            dp, q_scale, inv_tau, n_slots);                                                                          \
+        if (scan_waves == 1) FSIE_GLA_CHUNKS(T, 1);                                                                  \
+        else if (scan_waves == 2) FSIE_GLA_CHUNKS(T, 2);                                                             \
+        else if (scan_waves == 4) FSIE_GLA_CHUNKS(T, 4);                                                             \
+        else if (scan_waves == 8) FSIE_GLA_CHUNKS(T, 8);                                                             \
+        else FSIE_GLA_CHUNKS(T, 16);                                                                                 \
+    }
     if (dtype == FSIE_F32) {
         FSIE_GLA_BY_ROWS(float);
     } else {
@@ -202,6 +452,7 @@ extern "C" int fsie_gla_scan(const void* proj, int64_t proj_stride, int q_off, i
     }
 #undef FSIE_GLA_BY_ROWS
 #undef FSIE_GLA_LAUNCH
+#undef FSIE_GLA_CHUNKS
     FSIE_CHECK_LAUNCH("gla_scan");
     return 0;
 }

@@ -784,13 +784,15 @@ def softcap(x: torch.Tensor, cap: float) -> torch.Tensor:
 # ---------------------------------------------------------------------------------------------
 def gla_scan(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, z: torch.Tensor, state: torch.Tensor,
              q_starts: torch.Tensor, seq_slots: torch.Tensor, heads: int, dim: int, vdim: int, q_scale: float,
-             inv_tau: float) -> torch.Tensor:
+             inv_tau: float, chunked: bool = True) -> torch.Tensor:
     """S <- diag(sigmoid(z_t)^inv_tau) S + k_t v_t^T, o_t = S^T (q_scale q_t) over the tokens of every
     request of the step, from and to ``state`` float32 [slots, heads, dim, vdim].  ``proj`` [T, W] holds the
     q, k (heads x dim) and v (heads x vdim) columns from ``q_off``, ``k_off``, ``v_off``; ``z`` float32
     [T, heads * dim]; ``q_starts`` int32 [n + 1], ``seq_slots`` int32 [n].  Returns o float32 [P, T, heads * vdim]:
     the shares of the P groups of key channels that the kernel deals a head's state to (P follows from the
-    sizes alone); their sum in order is o, and ``gated_headnorm`` takes them as they are."""
+    sizes alone); their sum in order is o, and ``gated_headnorm`` takes them as they are.  Long portions are
+    computed chunk by chunk on the matrix cores (the same sums in another order); ``chunked=False`` walks
+    every portion token by token."""
     _need(proj, "gla proj", ndim=2)
     t, w = proj.shape
     _need(z, "gla z", dtype=torch.float32, shape=(t, heads * dim))
@@ -802,12 +804,18 @@ def gla_scan(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, z: torch.Te
     n = seq_slots.shape[0]
     if q_starts.shape[0] != n + 1:
         raise KernelError("gla: q_starts must have one entry more than seq_slots")
-    per_token, planes = ctypes.c_int(0), ctypes.c_int(0)
-    check(load().fsie_gla_scan_shape(heads, dim, vdim, ctypes.byref(per_token), ctypes.byref(planes)))
+    per_token, planes, chunk_tokens, chunk_min = ctypes.c_int(0), ctypes.c_int(0), ctypes.c_int(0), ctypes.c_int(0)
+    chunk_floats = ctypes.c_int64(0)
+    check(load().fsie_gla_scan_shape(heads, dim, vdim, ctypes.byref(per_token), ctypes.byref(planes),
+                                     ctypes.byref(chunk_tokens), ctypes.byref(chunk_min), ctypes.byref(chunk_floats)))
     prep = torch.empty((t * per_token.value,), dtype=torch.float32, device=proj.device)
     out = torch.empty((planes.value, t, heads * vdim), dtype=torch.float32, device=proj.device)
+    # a step of single tokens (t == n, as every captured decode step is) has no portion to cut into chunks
+    max_chunks = t // chunk_tokens.value + n if chunked and t > n and t >= chunk_min.value else 0
+    work = torch.empty((max_chunks * chunk_floats.value,), dtype=torch.float32, device=proj.device) if max_chunks else None
     check(load().fsie_gla_scan(proj.data_ptr(), w, q_off, k_off, v_off, z.data_ptr(), state.data_ptr(), q_starts.data_ptr(),
-                               seq_slots.data_ptr(), n, t, prep.data_ptr(), out.data_ptr(), heads, dim, vdim, float(q_scale),
+                               seq_slots.data_ptr(), n, t, prep.data_ptr(), out.data_ptr(),
+                               work.data_ptr() if work is not None else None, max_chunks, heads, dim, vdim, float(q_scale),
                                float(inv_tau), state.shape[0], dtype_code(proj.dtype), _stream()))
     return out
 

@@ -163,6 +163,53 @@ def test_gla_scan_over_portions_and_slots(ops, dtype, heads, dim, vdim):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("heads, dim, vdim, tau", [(2, 48, 40, 0.25), (1, 256, 200, 16.0), (5, 16, 64, 1.0), (2, 72, 130, 2.0)])
+def test_gla_scan_chunk_by_chunk_and_token_by_token(ops, dtype, heads, dim, vdim, tau):
+    """Portions around the length from which a portion is cut into chunks, whole chunks, one token more and one
+    less, a long one, beside single tokens; continued from a state that is not zero.  Decays of every kind in
+    one head: channels that forget everything within a token (their logarithms summed over a chunk are far
+    below what float32's exponential can hold) next to channels that keep everything, where a loud first token
+    must still be there at the end.  Both ways of walking a portion against the recurrence."""
+    scale = dim ** -0.5
+    lens = [[16, 15, 17, 1, 32, 250, 2, 33], [3, 250, 1, 16, 31, 40, 47, 1]]
+    kw, vw = heads * dim, heads * vdim
+    slots = [5, 0, 3, 1, 4, 7, 2, 6]
+    for chunked in (True, False):
+        state = torch.zeros(9, heads, dim, vdim).cuda()
+        datas, fed = [], [0] * len(slots)
+        for i in range(len(slots)):
+            n = lens[0][i] + lens[1][i]
+            proj, z = rnd((n, 2 * kw + vw), 30 + i).to(dtype), rnd((n, kw), 50 + i, 4.0)
+            z.view(n, heads, dim)[:, :, 0::3] = 25.0   # keeps everything
+            z.view(n, heads, dim)[:, :, 1::5] = -60.0  # keeps nothing
+            proj[0, kw:kw + kw] *= 30.0  # a loud first key: the keeping channels carry it to the last token
+            datas.append((proj, z))
+        outs = [[] for _ in slots]
+        for step in range(2):
+            rows = [(i, fed[i], fed[i] + lens[step][i]) for i in range(len(slots))]
+            proj = torch.cat([datas[i][0][lo:hi] for i, lo, hi in rows]).cuda()
+            z = torch.cat([datas[i][1][lo:hi] for i, lo, hi in rows]).cuda()
+            starts = np.cumsum([0] + [hi - lo for _, lo, hi in rows]).astype(np.int32)
+            o = ops.gla_scan(proj, 0, kw, 2 * kw, z, state, torch.from_numpy(starts).cuda(),
+                             torch.tensor(slots, dtype=torch.int32).cuda(), heads, dim, vdim, scale, 1 / tau, chunked=chunked)
+            assert torch.isfinite(o).all()
+            o = o.sum(0).cpu()
+            for i, lo, hi in rows:
+                outs[i].append(o[starts[i]:starts[i + 1]])
+                fed[i] = hi
+        for i, (proj, z) in enumerate(datas):
+            n, p = proj.shape[0], proj.double()
+            ref, final = oracle_gla_states(p[:, :kw].reshape(n, heads, dim) * scale, p[:, kw:2 * kw].reshape(n, heads, dim),
+                                           p[:, 2 * kw:].reshape(n, heads, vdim), z.double().reshape(n, heads, dim), tau,
+                                           torch.zeros(heads, dim, vdim, dtype=torch.float64))
+            got = torch.cat(outs[i]).reshape(n, heads, vdim)
+            assert rel(got, ref) <= 2e-5, (chunked, i)
+            assert rel(got[-1], ref[-1]) <= 2e-5, (chunked, i)
+            assert rel(state[slots[i]].cpu(), final) <= 2e-5, (chunked, i)
+        assert (state[8] == 0).all()
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_latent_prep_rope_pairs_and_head_gemm(ops, dtype):
     heads, q_rank, kv_rank, rot_dim, pairs, page, t = 3, 40, 52, 12, 4, 8, 11
     width = 64
