@@ -141,6 +141,86 @@ __global__ __launch_bounds__(kThreads) void head_gemm_kernel(const T* __restrict
     }
 }
 
+// The same product on the matrix cores, bfloat16 operands and float32 sums (v_mfma_f32_16x16x32_bf16): both x's
+// and w's rows run along K, which is what the instruction's operands want of a lane (eight neighbouring K
+// values of one row), so both are read from memory as they lie, no staging.  w is the first operand: a lane
+// then ends with four neighbouring outputs of one token, one 8-byte store.  A wave computes MT tiles of
+// sixteen tokens by four tiles of sixteen outputs; the four waves of a workgroup are next to each other along N.
+// Rows must start at multiples of eight values (16 bytes) and K must be one.
+typedef __bf16 hg_bf16x8 __attribute__((ext_vector_type(8)));
+typedef float hg_floatx4 __attribute__((ext_vector_type(4)));
+typedef unsigned hg_u32x4 __attribute__((ext_vector_type(4)));
+union HgFrag {
+    hg_u32x4 u;
+    hg_bf16x8 v;
+};
+
+template <int MT>
+__global__ __launch_bounds__(kThreads) void head_gemm_mfma_kernel(const bf16_t* __restrict__ x, int64_t x_stride, int x_off,
+                                                                  int x_hs, const bf16_t* __restrict__ w,
+                                                                  bf16_t* __restrict__ y, int64_t y_stride, int y_off,
+                                                                  int y_hs, const float* __restrict__ gate, int n_tokens,
+                                                                  int heads, int N, int K) {
+    const int h = blockIdx.z, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int n0 = (blockIdx.x * 4 + wave) * 64, t0 = blockIdx.y * (16 * MT);
+    if (n0 >= N) return;
+    const int r = lane & 15, kq = (lane >> 4) * 8;
+    const bf16_t* wh = w + static_cast<int64_t>(h) * N * K;
+    const bf16_t* wrow[4];
+    bool wok[4];
+#pragma unroll
+    for (int a = 0; a < 4; ++a) {
+        const int n = n0 + 16 * a + r;
+        wok[a] = n < N;
+        wrow[a] = wh + static_cast<int64_t>(min(n, N - 1)) * K + kq;
+    }
+    const bf16_t* xrow[MT];
+    bool xok[MT];
+#pragma unroll
+    for (int b = 0; b < MT; ++b) {
+        const int t = t0 + 16 * b + r;
+        xok[b] = t < n_tokens;
+        xrow[b] = x + static_cast<int64_t>(min(t, n_tokens - 1)) * x_stride + x_off + h * x_hs + kq;
+    }
+    hg_floatx4 acc[4][MT];
+#pragma unroll
+    for (int a = 0; a < 4; ++a) {
+#pragma unroll
+        for (int b = 0; b < MT; ++b) acc[a][b] = hg_floatx4{0.f, 0.f, 0.f, 0.f};
+    }
+    const hg_u32x4 zero = {0u, 0u, 0u, 0u};
+    for (int k0 = 0; k0 < K; k0 += 32) {
+        const bool kok = k0 + kq < K;  // K is a multiple of eight: a lane's eight values are all inside or all outside
+        HgFrag wf[4], xf[MT];
+#pragma unroll
+        for (int a = 0; a < 4; ++a) wf[a].u = (kok && wok[a]) ? *reinterpret_cast<const hg_u32x4*>(wrow[a] + k0) : zero;
+#pragma unroll
+        for (int b = 0; b < MT; ++b) xf[b].u = (kok && xok[b]) ? *reinterpret_cast<const hg_u32x4*>(xrow[b] + k0) : zero;
+#pragma unroll
+        for (int a = 0; a < 4; ++a) {
+#pragma unroll
+            for (int b = 0; b < MT; ++b) acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[a].v, xf[b].v, acc[a][b], 0, 0, 0);
+        }
+    }
+    // lane: the outputs 4 (lane / 16) .. + 3 of a tile of sixteen, of the token lane % 16 of a tile
+    const int nq = (lane >> 4) * 4;
+#pragma unroll
+    for (int b = 0; b < MT; ++b) {
+        const int t = t0 + 16 * b + r;
+        if (t >= n_tokens) continue;
+        const float g = gate ? gate[static_cast<int64_t>(t) * heads + h] : 1.0f;
+        bf16_t* dst = y + static_cast<int64_t>(t) * y_stride + y_off + h * y_hs;
+#pragma unroll
+        for (int a = 0; a < 4; ++a) {
+            const int n = n0 + 16 * a + nq;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                if (n + i < N) dst[n + i] = from_float<bf16_t>(acc[a][b][i] * g);
+            }
+        }
+    }
+}
+
 }  // namespace
 
 extern "C" int fsie_latent_prep(const void* proj, int64_t stride, int dq_off, int q_rank, int dkv_off, int kv_rank,
@@ -213,7 +293,23 @@ extern "C" int fsie_head_gemm(const void* x, int64_t x_stride, int x_off, int x_
     const int row_tiles = (n_tokens + kTileM - 1) / kTileM;
     FSIE_REQUIRE(row_tiles <= 65535, "head_gemm: %d tokens are more than one launch takes", n_tokens);
     const dim3 grid((N + kTileN - 1) / kTileN, row_tiles, heads);
-    if (dtype == FSIE_F32) {
+    const bool aligned = K % 8 == 0 && x_stride % 8 == 0 && x_off % 8 == 0 && x_hs % 8 == 0 &&
+                         reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(w) % 16 == 0;
+    if (dtype == FSIE_BF16 && aligned) {
+        const bool two = n_tokens > 16;
+        const int token_tiles = (n_tokens + (two ? 32 : 16) - 1) / (two ? 32 : 16);
+        FSIE_REQUIRE(token_tiles <= 65535, "head_gemm: %d tokens are more than one launch takes", n_tokens);
+        const dim3 mgrid((N + 255) / 256, token_tiles, heads);
+        if (two) {
+            head_gemm_mfma_kernel<2><<<mgrid, kThreads, 0, stream>>>(static_cast<const bf16_t*>(x), x_stride, x_off, x_hs,
+                                                                    static_cast<const bf16_t*>(w), static_cast<bf16_t*>(y),
+                                                                    y_stride, y_off, y_hs, gate, n_tokens, heads, N, K);
+        } else {
+            head_gemm_mfma_kernel<1><<<mgrid, kThreads, 0, stream>>>(static_cast<const bf16_t*>(x), x_stride, x_off, x_hs,
+                                                                    static_cast<const bf16_t*>(w), static_cast<bf16_t*>(y),
+                                                                    y_stride, y_off, y_hs, gate, n_tokens, heads, N, K);
+        }
+    } else if (dtype == FSIE_F32) {
         head_gemm_kernel<float><<<grid, kThreads, 0, stream>>>(static_cast<const float*>(x), x_stride, x_off, x_hs,
                                                              static_cast<const float*>(w), static_cast<float*>(y), y_stride,
                                                              y_off, y_hs, gate, n_tokens, heads, N, K);

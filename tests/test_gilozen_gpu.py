@@ -265,6 +265,27 @@ def test_latent_prep_rope_pairs_and_head_gemm(ops, dtype):
     assert rel(y.float().cpu().reshape(t, heads, 9), ref) <= tol(dtype, bf16=2.0 ** -7)
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("t, heads, k, n", [(5, 3, 8, 9), (16, 2, 40, 64), (17, 1, 64, 200), (100, 5, 96, 300), (33, 2, 24, 17)])
+def test_head_gemm_on_rows_that_the_matrix_cores_take(ops, dtype, t, heads, k, n):
+    """Heads whose values start at multiples of eight columns (the matrix-core kernel's condition in bfloat16):
+    token counts around its tiles of sixteen and thirty-two, outputs that do not fill a tile or a wave, a K
+    that is not a multiple of the instruction's thirty-two, gaps between the heads in x and in out, a gate; the
+    columns of out that belong to no head stay as they were."""
+    x_off, x_hs, out_off, out_hs = 16, k + 8, 3, n + 2
+    x = rnd((t, x_off + heads * x_hs + 8), t).to(dtype)
+    w = rnd((heads, n, k), n, k ** -0.5).to(dtype)
+    gate = torch.sigmoid(rnd((t, heads), 3))
+    for g in (None, gate):
+        out = torch.full((t, out_off + heads * out_hs), 5.0, dtype=dtype).cuda()
+        ops.head_gemm(x.cuda(), x_off, x_hs, w.cuda(), out, out_off, out_hs, gate=None if g is None else g.cuda())
+        xs = x.double()[:, x_off:x_off + heads * x_hs].reshape(t, heads, x_hs)[..., :k]
+        ref = torch.einsum("thk,hnk->thn", xs, w.double()) * (1.0 if g is None else g.double().unsqueeze(-1))
+        got = out.float().cpu()
+        assert rel(got[:, out_off:].reshape(t, heads, out_hs)[..., :n], ref) <= tol(dtype, f32=1e-5, bf16=2.0 ** -7)
+        assert (got[:, :out_off] == 5.0).all() and (got[:, out_off:].reshape(t, heads, out_hs)[..., n:] == 5.0).all()
+
+
 def attention_with_sinks(ops, case, heads, hd, sinks, scale, share_keys=True):
     from from_scratch_inference_engine_amd.parts.attention import paged_attention
 
