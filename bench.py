@@ -278,7 +278,8 @@ def design_comparison(args) -> int:
                 "rms_norm_eps": 1e-5, "tie_word_embeddings": False, "max_position_embeddings": 8192}
         for name, raw in (("gilozen", gilozen_shape(width, ff, layers, vocab)), ("qwen2", qwen)):
             model = Model.from_random(parse_config(raw), seed=0, dtype=dtype)
-            runner = Runner(model, page_size=16, num_pages=64 * 40 + 160, max_requests=64)
+            pages_each = (512 + args.warmup + args.steps) // 16 + 2  # a decoding request's context and every step after it
+            runner = Runner(model, page_size=16, num_pages=64 * max(40, pages_each) + 160, max_requests=64)
             row = {"weights_gb": model.weight_bytes / 1e9}
             times = []
             for rep in range(4 if "prefill" in phases else 0):

@@ -161,14 +161,17 @@ __device__ __forceinline__ int gla_chunks_of(const int32_t* q_starts, const int3
 // channels past dim count as decay 1 with q = k = 0.
 __host__ __device__ inline int64_t gla_chunk_floats(int dp) { return static_cast<int64_t>(2 * kGlaChunk + 1) * dp + kGlaChunk * kGlaChunk; }
 
-// grid = (upper bound of the step's chunks, heads).
+// grid = (upper bound of the step's chunks, heads).  The logarithms are kept to the base two (the hardware's
+// exponential is 2^x).  Every (token, channel) of the chunk is one thread's in the loads and in the stores; only
+// the running sums over the chunk's tokens are a thread a channel.  A's pairs (j <= i) are dealt to the first
+// 136 threads, row i together with row 15 - i, so that no wave carries the empty half of the square.
 template <typename T>
 __global__ __launch_bounds__(kGlaChunkThreads) void gla_chunk_prep_kernel(
     const T* __restrict__ proj, int64_t proj_stride, int q_off, int k_off, const float* __restrict__ z,
     float* __restrict__ work, const int32_t* __restrict__ q_starts, const int32_t* __restrict__ seq_slots, int n_seqs,
     int heads, int dim, int dp, float q_scale, float inv_tau, int n_slots) {
-    extern __shared__ float lds[];  // [3][16][dp + 1]: q, k, B
-    const int ld = dp + 1;
+    extern __shared__ float lds[];  // [3][16][dp + 4]: q, k, B
+    const int ld = dp + 4;
     float* qs = lds;
     float* ks = qs + kGlaChunk * ld;
     float* bs = ks + kGlaChunk * ld;
@@ -187,43 +190,67 @@ __global__ __launch_bounds__(kGlaChunkThreads) void gla_chunk_prep_kernel(
     float* kdT = qd + kGlaChunk * dp;
     float* g = kdT + kGlaChunk * dp;
     float* A = g + dp;
+    const float to_log2 = inv_tau * 1.44269504088896340736f;
 
+    for (int e = tid; e < kGlaChunk * dp; e += kGlaChunkThreads) {
+        const int t = e / dp, c = e - t * dp;
+        float q = 0.f, k = 0.f, la = 0.f;
+        if (t < nt && c < dim) {
+            const T* row = proj + static_cast<int64_t>(t0 + t) * proj_stride + h * dim + c;
+            q = to_float(row[q_off]) * q_scale;
+            k = to_float(row[k_off]);
+            la = to_log2 * log_sigmoid(z[(static_cast<int64_t>(t0 + t) * heads + h) * dim + c]);
+        }
+        qs[t * ld + c] = q;
+        ks[t * ld + c] = k;
+        bs[t * ld + c] = la;
+    }
+    __syncthreads();
     for (int c = tid; c < dp; c += kGlaChunkThreads) {
-        float q[kGlaChunk], k[kGlaChunk], b[kGlaChunk];
         float sum = 0.f;
 #pragma unroll
         for (int t = 0; t < kGlaChunk; ++t) {
-            q[t] = 0.f;
-            k[t] = 0.f;
-            if (t < nt && c < dim) {
-                const T* row = proj + static_cast<int64_t>(t0 + t) * proj_stride + h * dim + c;
-                q[t] = to_float(row[q_off]) * q_scale;
-                k[t] = to_float(row[k_off]);
-                sum += inv_tau * log_sigmoid(z[(static_cast<int64_t>(t0 + t) * heads + h) * dim + c]);
-            }
-            b[t] = sum;
-            qs[t * ld + c] = q[t];
-            ks[t * ld + c] = k[t];
+            sum += bs[t * ld + c];
             bs[t * ld + c] = sum;
         }
-        floatx4 kd[kGlaChunk / 4];
-#pragma unroll
-        for (int t = 0; t < kGlaChunk; ++t) {
-            qd[t * dp + c] = q[t] * expf(b[t]);
-            kd[t / 4][t % 4] = k[t] * expf(sum - b[t]);
-        }
-#pragma unroll
-        for (int t4 = 0; t4 < kGlaChunk / 4; ++t4) *reinterpret_cast<floatx4*>(kdT + c * kGlaChunk + 4 * t4) = kd[t4];
-        g[c] = expf(sum);
+        g[c] = __builtin_amdgcn_exp2f(sum);
     }
     __syncthreads();
-    for (int e = tid; e < kGlaChunk * kGlaChunk; e += kGlaChunkThreads) {
-        const int i = e / kGlaChunk, j = e % kGlaChunk;
+    for (int e = tid; e < kGlaChunk * dp; e += kGlaChunkThreads) {
+        const int t = e / dp, c = e - t * dp;
+        qd[e] = qs[t * ld + c] * __builtin_amdgcn_exp2f(bs[t * ld + c]);
+    }
+    for (int e = tid; e < dp * (kGlaChunk / 4); e += kGlaChunkThreads) {
+        const int c = e >> 2, t4 = (e & 3) * 4;
+        const float last = bs[(kGlaChunk - 1) * ld + c];
+        floatx4 kd;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) kd[i] = ks[(t4 + i) * ld + c] * __builtin_amdgcn_exp2f(last - bs[(t4 + i) * ld + c]);
+        *reinterpret_cast<floatx4*>(kdT + c * kGlaChunk + t4) = kd;
+    }
+    // A: thread p < 136 has the pair number p of the rows (r, 15 - r) put side by side, r = p / 17
+    if (tid < kGlaChunk * (kGlaChunk + 1) / 2) {
+        const int r = tid / (kGlaChunk + 1), o = tid - r * (kGlaChunk + 1);
+        const int i = o <= r ? r : kGlaChunk - 1 - r;
+        const int j = o <= r ? o : o - r - 1;
         float a = 0.f;
-        if (j <= i && i < nt) {
-            for (int c = 0; c < dim; ++c) a = fmaf(qs[i * ld + c] * ks[j * ld + c], expf(bs[i * ld + c] - bs[j * ld + c]), a);
+        if (i < nt) {
+            const float* qi = qs + i * ld;
+            const float* kj = ks + j * ld;
+            const float* bi = bs + i * ld;
+            const float* bj = bs + j * ld;
+            for (int c = 0; c < dp; c += 4) {  // (channels past dim: q = k = 0)
+                const floatx4 q4 = *reinterpret_cast<const floatx4*>(qi + c), k4 = *reinterpret_cast<const floatx4*>(kj + c);
+                const floatx4 x4 = *reinterpret_cast<const floatx4*>(bi + c) - *reinterpret_cast<const floatx4*>(bj + c);
+#pragma unroll
+                for (int u = 0; u < 4; ++u) a = fmaf(q4[u] * k4[u], __builtin_amdgcn_exp2f(x4[u]), a);
+            }
         }
-        A[e] = a;
+        A[i * kGlaChunk + j] = a;
+    }
+    // above the diagonal: zeros
+    for (int e = tid; e < kGlaChunk * kGlaChunk; e += kGlaChunkThreads) {
+        if ((e & 15) > (e >> 4)) A[e] = 0.f;
     }
 }
 
@@ -415,7 +442,7 @@ extern "C" int fsie_gla_scan(const void* proj, int64_t proj_stride, int q_off, i
     }
     const int skip_from = chunks ? kGlaChunkMin : 0x7fffffff;
     const dim3 chunk_grid(chunks ? max_chunks : 1, heads);
-    const size_t chunk_lds = 3 * kGlaChunk * (dp + 1) * sizeof(float);
+    const size_t chunk_lds = 3 * kGlaChunk * (dp + 4) * sizeof(float);
     const dim3 scan_grid(n_seqs, heads, (vdim + 15) / 16);
     int scan_waves = 1;  // a wave for every sixteen key channels, rounded up to a power of two: at most sixteen
     while (scan_waves * 16 < dim) scan_waves *= 2;

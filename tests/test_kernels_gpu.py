@@ -564,10 +564,10 @@ def test_refusals(ops):
     with pytest.raises(KernelError, match="float32 or bfloat16"):
         ops.swiglu(torch.zeros(2, 4, dtype=torch.float16).cuda())
     with pytest.raises(KernelError, match="head_dim"):
-        q = torch.zeros(1, 3 * 300).cuda()
-        ops.attention_scalar(q, 900, torch.zeros(1, 1, 4, 300).cuda(), torch.zeros(1, 1, 300, 4).cuda(),
+        q = torch.zeros(1, 3 * 600).cuda()  # (heads of up to 512 values have a kernel)
+        ops.attention_scalar(q, 1800, torch.zeros(1, 1, 4, 600).cuda(), torch.zeros(1, 1, 600, 4).cuda(),
                              torch.zeros(1, 1, dtype=torch.int32).cuda(), torch.zeros(1, 8, dtype=torch.int32).cuda(), 1,
-                             torch.zeros(1, 300).cuda(), None, 1, 1, 300, None, 1.0, 1)
+                             torch.zeros(1, 600).cuda(), None, 1, 1, 600, None, 1.0, 1)
 
 
 # ------------------------------------------------------------------------------ attention
