@@ -52,12 +52,19 @@ __device__ __forceinline__ float log_sigmoid(float z) { return fminf(z, 0.f) - l
 // trips to memory, ten times its arithmetic.  What the waves exchange here goes through shared memory alone.
 __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
-// prep [3][tokens][heads][dp]: scaled q, k, decay.
+// prep [3][tokens][heads][dp]: scaled q, k, decay.  Grid: blocks of 256 elements over all tokens of the step,
+// or (with short_only > 0) over the first tokens of every request (grid.y), and only for requests of at most
+// short_only tokens: the others go chunk by chunk and need none of this.
 template <typename T>
 __global__ void gla_prep_kernel(const T* __restrict__ proj, int64_t proj_stride, int q_off, int k_off,
                                 const float* __restrict__ z, float* __restrict__ prep, int64_t total, int heads, int dim,
-                                int dp, float q_scale, float inv_tau) {
-    const int64_t e = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+                                int dp, float q_scale, float inv_tau, const int32_t* __restrict__ q_starts, int short_only) {
+    int64_t e = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (short_only > 0) {
+        const int lo = q_starts[blockIdx.y], len = q_starts[blockIdx.y + 1] - lo;
+        if (len > short_only || e >= static_cast<int64_t>(len) * heads * dp) return;
+        e += static_cast<int64_t>(lo) * heads * dp;
+    }
     if (e >= total) return;
     const int i = static_cast<int>(e % dp);
     const int64_t th = e / dp;
@@ -432,7 +439,6 @@ extern "C" int fsie_gla_scan(const void* proj, int64_t proj_stride, int q_off, i
     FSIE_REQUIRE(heads <= 65535 && col_blocks * splits <= 65535 && (vdim + 15) / 16 <= 65535, "gla_scan: too many heads or columns");
     const int64_t plane = static_cast<int64_t>(n_tokens) * heads * dp;
     const int64_t out_plane = static_cast<int64_t>(n_tokens) * heads * vdim;
-    const unsigned prep_grid = static_cast<unsigned>(ceil_div64(plane, 256));
     const dim3 grid(n_seqs, heads, col_blocks * splits);
     const bool chunks = chunk_work != nullptr && n_tokens >= kGlaChunkMin;
     if (chunks) {
@@ -441,6 +447,12 @@ extern "C" int fsie_gla_scan(const void* proj, int64_t proj_stride, int q_off, i
         FSIE_REQUIRE(max_chunks <= 0x7fffffff / kGlaChunk, "gla_scan: too many chunks");
     }
     const int skip_from = chunks ? kGlaChunkMin : 0x7fffffff;
+    // with the chunk kernels at work only portions below their length are walked: their first tokens, request by request
+    const int short_only = chunks ? kGlaChunkMin - 1 : 0;
+    const dim3 prep_grid(static_cast<unsigned>(chunks ? ceil_div64(static_cast<int64_t>(short_only) * heads * dp, 256)
+                                                      : ceil_div64(plane, 256)),
+                         chunks ? n_seqs : 1);
+    FSIE_REQUIRE(n_seqs <= 65535 || !chunks, "gla_scan: too many requests");
     const dim3 chunk_grid(chunks ? max_chunks : 1, heads);
     const size_t chunk_lds = 3 * kGlaChunk * (dp + 4) * sizeof(float);
     const dim3 scan_grid(n_seqs, heads, (vdim + 15) / 16);
@@ -456,7 +468,7 @@ extern "C" int fsie_gla_scan(const void* proj, int64_t proj_stride, int q_off, i
                                                                dp, splits, n_slots, skip_from)
 #define FSIE_GLA_BY_ROWS(T)                                                                                          \
     gla_prep_kernel<T><<<prep_grid, 256, 0, stream>>>(static_cast<const T*>(proj), proj_stride, q_off, k_off, z, prep, \
-                                                      plane, heads, dim, dp, q_scale, inv_tau);                      \
+                                                      plane, heads, dim, dp, q_scale, inv_tau, q_starts, short_only); \
     if (rows == 1) FSIE_GLA_LAUNCH(T, 1);                                                                            \
     else if (rows == 2) FSIE_GLA_LAUNCH(T, 2);                                                                       \
     else if (rows == 4) FSIE_GLA_LAUNCH(T, 4);                                                                       \

@@ -275,7 +275,7 @@ def test_graft_entry_smoke():
 def test_bench_prints_its_line():
     """bench.py as it is run for the record, at a small shape (two layers of 896 / 4864): the library's
     kernels chosen by timing, prefill, decode at batch 8, 1 and 64 through the engine, the time of each
-    class of kernels; one JSON line with the fields of the contract.  More than one GPU: one line, exit 2."""
+    class of kernels; one JSON line with the fields that a benchmark driver reads.  More than one GPU: one line, exit 2."""
     cmd = [sys.executable, "bench.py", "--shape", "0.5b", "--layers", "2", "--steps", "8", "--warmup", "4"]
     proc = subprocess.run(cmd, capture_output=True, text=True, timeout=300, cwd=str(helpers.ROOT))
     assert proc.returncode == 0, proc.stderr[-3000:]
