@@ -428,7 +428,17 @@ CONFIG_C = {"architecture": "Gilozen", "width": 64, "vocab": 150, "norm": {"eps"
     layer("latent_attention", latent(2, 16, 16, 24, 270, 48), 96),
     layer("gla", {"heads": 2, "dim": 16, "vdim": 32, "tau": 4.0}, 96),
 ]}
-DECAY_RANK = {"A": 12, "B": 8, "C": 4}
+# D: linear attention only (no paged cache at all); E: attention only (no state slots), the last layer borrowing
+CONFIG_D = {"architecture": "Gilozen", "width": 48, "vocab": 97, "norm": {"eps": 1e-5}, "logit_softcap": 9.0, "layers": [
+    layer("gla", {"heads": 2, "dim": 24, "vdim": 40, "tau": 3.0}, 64),
+    layer("gla", {"heads": 1, "dim": 40, "vdim": 24, "tau": 1.0}, None),
+]}
+CONFIG_E = {"architecture": "Gilozen", "width": 56, "vocab": 120, "norm": {"eps": 1e-6}, "layers": [
+    layer("latent_attention", latent(2, 16, 8, 24, 40, 32), None),
+    layer("latent_attention", latent(4, 8, 16, 8, 24, 16, base=100.0), 80),
+    layer("latent_attention", latent(3, 24, 8, 16, 40, 48, kv_from=0), 48),
+]}
+DECAY_RANK = {"A": 12, "B": 8, "C": 4, "D": 6, "E": 1}
 
 
 def gilozen_tensors(cfg, rank, seed):
@@ -471,7 +481,7 @@ def gilozen_tensors(cfg, rank, seed):
 def models(tmp_path_factory):
     root = tmp_path_factory.mktemp("gilozen")
     out = {}
-    for name, cfg in (("A", CONFIG_A), ("B", CONFIG_B), ("C", CONFIG_C)):
+    for name, cfg in (("A", CONFIG_A), ("B", CONFIG_B), ("C", CONFIG_C), ("D", CONFIG_D), ("E", CONFIG_E)):
         d = helpers.make_model_dir(root / name, cfg, 0, tensors=gilozen_tensors(cfg, DECAY_RANK[name], seed=len(name) + ord(name)))
         out[name] = (d, plain.read_config(d), plain.read_weights(d))
     return out
@@ -556,6 +566,28 @@ def test_model_whole_in_portions_decoded_and_batched(models, name, dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["D", "E"])
+def test_model_of_one_kind_of_layer(models, name, dtype):
+    """A model with state slots and no paged cache, and one with a paged cache and no state: whole, a portion and
+    then token by token, and two requests of unequal length together, in a pool that is used again."""
+    from from_scratch_inference_engine_amd import load_model
+    from from_scratch_inference_engine_amd.engine.model import Runner
+
+    d, cfg, w = models[name]
+    seqs = {"a": helpers.token_ids(cfg["vocab"], 70, 1), "b": helpers.token_ids(cfg["vocab"], 23, 2)}
+    ref = {r: plain.forward(cfg, w, ids).numpy() for r, ids in seqs.items()}
+    runner = Runner(load_model(d, dtype=dtype), page_size=8, num_pages=14, max_requests=2)
+    got = step_through(runner, [[(r, len(ids))] for r, ids in seqs.items()], seqs)
+    for r in seqs:
+        close_enough(got[r], ref[r], dtype, f"{name} whole {r}")
+    got = step_through(runner, [[("a", 37)]] + [[("a", 1)]] * 33, {"a": seqs["a"]})
+    close_enough(got["a"], ref["a"], dtype, f"{name} decode")
+    got = step_through(runner, [[("a", 50), ("b", 2)], [("a", 19), ("b", 1)], [("a", 1), ("b", 17)], [("b", 3)]], seqs)
+    for r in seqs:
+        close_enough(got[r], ref[r], dtype, f"{name} batched {r}")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_model_with_cache_rows_beyond_256_values(models, dtype):
     from from_scratch_inference_engine_amd import load_model
     from from_scratch_inference_engine_amd.engine.model import Runner
@@ -592,9 +624,11 @@ def test_greedy_generation_through_the_engine(models, name):
     assert llm.engine.runner.graphs.replays > 0
 
 
-def test_replay_program_runs_the_model(models, tmp_path):
-    """bin/trace_run on the architecture: a prompt in portions beside another request's single tokens."""
-    d, cfg, w = models["A"]
+@pytest.mark.parametrize("name", ["A", "D", "E"])
+def test_replay_program_runs_the_model(models, tmp_path, name):
+    """bin/trace_run on the architecture (mixed layers, state only, cache only): a prompt in portions beside
+    another request's single tokens."""
+    d, cfg, w = models[name]
     a, b = helpers.token_ids(cfg["vocab"], 50, 7), helpers.token_ids(cfg["vocab"], 20, 8)
     tb = helpers.TraceBuilder()
     tb.step([("a", a[:17], [16]), ("b", b[:1], [0])])
