@@ -298,7 +298,7 @@ __global__ __launch_bounds__(64 * NW) void gla_chunk_scan_kernel(
     }
     const int64_t per_chunk = gla_chunk_floats(dp) * heads;
     const float* w = work + (static_cast<int64_t>(first) * heads + h) * gla_chunk_floats(dp);
-    const T* vp = proj + v_off + h * vdim + min(col, vdim - 1);  // (columns past the head's last: a number, unused)
+    const T* vp = proj + v_off + h * vdim;
     const int64_t out_stride = static_cast<int64_t>(heads) * vdim;
 
     // The operands of the next D - 1 chunks are on their way while a chunk is multiplied: a ring of D sets of
@@ -306,19 +306,57 @@ __global__ __launch_bounds__(64 * NW) void gla_chunk_scan_kernel(
     constexpr int D = 4;
     floatx4 q4[D], k4[D], g4v[D], a4[D];
     float v[D][4];
+    // A chunk's addresses are a base that is the same in all lanes plus a lane's share that never changes.
+    const int q_at = n * dp + ch0 + 4 * g4;
+    const int k_at = kGlaChunk * dp + (ch0 + n) * kGlaChunk + 4 * g4;
+    const int g_at = 2 * kGlaChunk * dp + ch0 + 4 * g4;
+    const int a_at = (2 * kGlaChunk + 1) * dp + n * kGlaChunk + 4 * g4;
+    const int v_col = min(col, vdim - 1);  // (columns past the head's last: a number, unused)
+    int v_at[4];
+#pragma unroll
+    for (int m = 0; m < 4; ++m) v_at[m] = (4 * g4 + m) * static_cast<int>(proj_stride) + v_col;
     auto fetch = [&](const int slot_, int ci) {
         ci = min(ci, n_chunks - 1);  // past the end: the last chunk once more, never used
         const float* wc = w + ci * per_chunk;
         const int t0 = lo + ci * kGlaChunk;
+        const T* vc = vp + static_cast<int64_t>(t0) * proj_stride;
+        // (a token past the portion's end has q = k = 0 and a zero row and column of A: the v of the portion's
+        // last token stands in for it, a number that is multiplied by zero)
+        if (t0 + kGlaChunk <= hi) {  // the same in all lanes
 #pragma unroll
-        for (int m = 0; m < 4; ++m) {
-            const int t = min(t0 + 4 * g4 + m, hi - 1);
-            v[slot_][m] = to_float(vp[static_cast<int64_t>(t) * proj_stride]);
+            for (int m = 0; m < 4; ++m) v[slot_][m] = to_float(vc[v_at[m]]);
+        } else {
+#pragma unroll
+            for (int m = 0; m < 4; ++m) {
+                v[slot_][m] = to_float(vc[static_cast<int64_t>(min(4 * g4 + m, hi - 1 - t0)) * proj_stride + v_col]);
+            }
         }
-        q4[slot_] = *reinterpret_cast<const floatx4*>(wc + n * dp + ch0 + 4 * g4);
-        k4[slot_] = *reinterpret_cast<const floatx4*>(wc + kGlaChunk * dp + (ch0 + n) * kGlaChunk + 4 * g4);
-        g4v[slot_] = *reinterpret_cast<const floatx4*>(wc + 2 * kGlaChunk * dp + ch0 + 4 * g4);
-        a4[slot_] = *reinterpret_cast<const floatx4*>(wc + (2 * kGlaChunk + 1) * dp + n * kGlaChunk + 4 * g4);
+        q4[slot_] = *reinterpret_cast<const floatx4*>(wc + q_at);
+        k4[slot_] = *reinterpret_cast<const floatx4*>(wc + k_at);
+        g4v[slot_] = *reinterpret_cast<const floatx4*>(wc + g_at);
+        a4[slot_] = *reinterpret_cast<const floatx4*>(wc + a_at);
+    };
+    // o of chunk ci from the waves' shares, added in the order of the waves (the first 256 threads, one value
+    // each; with fewer threads, several).  Further planes of `out`: zeros.
+    auto finish = [&](int ci, bool really) {
+        const int t0 = lo + ci * kGlaChunk;
+        float* oc = out + static_cast<int64_t>(t0) * out_stride + h * vdim + blockIdx.z * 16;
+#pragma unroll
+        for (int e0 = 0; e0 < 256; e0 += 64 * NW) {
+            const int e = e0 + tid;
+            if (e < 256) {
+                const int i = e >> 6, l = e & 63;
+                float sum = part[ci & 1][0][i][l];
+#pragma unroll
+                for (int ww = 1; ww < NW; ++ww) sum += part[ci & 1][ww][i][l];
+                const int tok = 4 * (l >> 4) + i, c = l & 15;
+                if (really && t0 + tok < hi && blockIdx.z * 16 + c < vdim) {
+                    float* dst = oc + tok * static_cast<int>(out_stride) + c;
+                    *dst = sum;
+                    for (int pl = 1; pl < planes; ++pl) dst[pl * out_plane] = 0.f;
+                }
+            }
+        }
     };
 #pragma unroll
     for (int u = 0; u < D - 1; ++u) fetch(u, u);
@@ -329,47 +367,32 @@ __global__ __launch_bounds__(64 * NW) void gla_chunk_scan_kernel(
             if (ci < n_chunks) {  // the same for the whole workgroup
                 fetch((u + D - 1) % D, ci + D - 1);
                 const int t0 = lo + ci * kGlaChunk;
-                // (a token past the portion's end has k = 0 and a zero row of A: whatever v was read for it
-                // is multiplied by zero, but it must be a number)
-                float cv[4];
-#pragma unroll
-                for (int m = 0; m < 4; ++m) cv[m] = (t0 + 4 * g4 + m < hi && col_ok) ? v[u][m] : 0.f;
-                floatx4 o[4];
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    o[i] = __builtin_amdgcn_mfma_f32_16x16x4f32(q4[u][i], S[i], floatx4{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
-                }
+                // o in two sums that do not wait for each other
+                const floatx4 zero = {0.f, 0.f, 0.f, 0.f};
+                floatx4 o[2];
+                o[0] = __builtin_amdgcn_mfma_f32_16x16x4f32(q4[u][0], S[0], zero, 0, 0, 0);
+                o[1] = __builtin_amdgcn_mfma_f32_16x16x4f32(q4[u][1], S[1], zero, 0, 0, 0);
+                o[0] = __builtin_amdgcn_mfma_f32_16x16x4f32(q4[u][2], S[2], o[0], 0, 0, 0);
+                o[1] = __builtin_amdgcn_mfma_f32_16x16x4f32(q4[u][3], S[3], o[1], 0, 0, 0);
 #pragma unroll
                 for (int m = 0; m < 4; ++m) {
-                    if (m % NW == wave) o[m] = __builtin_amdgcn_mfma_f32_16x16x4f32(a4[u][m], cv[m], o[m], 0, 0, 0);
+                    if (m % NW == wave) o[m & 1] = __builtin_amdgcn_mfma_f32_16x16x4f32(a4[u][m], v[u][m], o[m & 1], 0, 0, 0);
                 }
                 S *= g4v[u];
 #pragma unroll
-                for (int m = 0; m < 4; ++m) S = __builtin_amdgcn_mfma_f32_16x16x4f32(k4[u][m], cv[m], S, 0, 0, 0);
-                const floatx4 mine = (o[0] + o[1]) + (o[2] + o[3]);
+                for (int m = 0; m < 4; ++m) S = __builtin_amdgcn_mfma_f32_16x16x4f32(k4[u][m], v[u][m], S, 0, 0, 0);
+                // the chunk before this one: its shares lie in the other half of `part` since the last barrier;
+                // adding them up and storing o goes on while the matrix instructions above are at work
+                finish(ci - 1, ci > 0);
+                const floatx4 mine = o[0] + o[1];
 #pragma unroll
                 for (int i = 0; i < 4; ++i) part[ci & 1][wave][i][lane] = mine[i];
+                // everyone has written this chunk's half and has read the other: the next chunk may overwrite that
                 lds_barrier();
-                // (the barrier of the next chunk keeps its writers off this half until everyone has read it)
-#pragma unroll
-                for (int e0 = 0; e0 < 256; e0 += 64 * NW) {
-                    const int e = e0 + tid;
-                    if (e < 256) {
-                        const int i = e >> 6, l = e & 63;
-                        float sum = part[ci & 1][0][i][l];
-#pragma unroll
-                        for (int ww = 1; ww < NW; ++ww) sum += part[ci & 1][ww][i][l];
-                        const int t = t0 + 4 * (l >> 4) + i, cc = blockIdx.z * 16 + (l & 15);
-                        if (t < hi && cc < vdim) {
-                            float* dst = out + static_cast<int64_t>(t) * out_stride + h * vdim + cc;
-                            *dst = sum;
-                            for (int pl = 1; pl < planes; ++pl) dst[pl * out_plane] = 0.f;
-                        }
-                    }
-                }
             }
         }
     }
+    finish(n_chunks - 1, true);
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         const int row = ch0 + 4 * g4 + i;
@@ -445,6 +468,8 @@ extern "C" int fsie_gla_scan(const void* proj, int64_t proj_stride, int q_off, i
         FSIE_REQUIRE(max_chunks >= n_tokens / kGlaChunk + n_seqs, "gla_scan: room for %d chunks, the step may have %d",
                      max_chunks, n_tokens / kGlaChunk + n_seqs);
         FSIE_REQUIRE(max_chunks <= 0x7fffffff / kGlaChunk, "gla_scan: too many chunks");
+        FSIE_REQUIRE(proj_stride <= 0x7fffffff / kGlaChunk && static_cast<int64_t>(heads) * vdim <= 0x7fffffff / kGlaChunk,
+                     "gla_scan: rows too long for the chunk kernels' 32-bit offsets");
     }
     const int skip_from = chunks ? kGlaChunkMin : 0x7fffffff;
     // with the chunk kernels at work only portions below their length are walked: their first tokens, request by request
