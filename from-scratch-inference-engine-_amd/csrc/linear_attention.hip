@@ -24,8 +24,8 @@
 // q and k, the chunk's decay and A for every chunk and head at once (float32 on the vector units); the walk
 // over chunks then is three small matrix products a chunk on the float32 matrix instruction
 // (v_mfma_f32_16x16x4_f32, no rounding of operands), one wave per sixteen key channels and sixteen value
-// columns with its tile of S in an accumulator; the waves of a head's columns meet once a chunk to add their
-// shares of o.
+// columns with its tile of S in an accumulator; the waves of a head's columns meet every few chunks to add
+// their shares of o.
 #include "common.h"
 #include "api.h"
 
@@ -267,15 +267,16 @@ __global__ __launch_bounds__(kGlaChunkThreads) void gla_chunk_prep_kernel(
 // the instruction's second operand over four steps, if step i takes the channels 4 g + i (g = 0..3) as its four
 // inner indices; a sum does not mind the order, so S is multiplied from the left as it lies.  The same
 // renumbering of the inner index (the tokens 4 g + m at step m) lets v, kdT and A be read in vectors of four.
-// A wave's chain per chunk is nine matrix instructions; the waves' shares of the chunk's o (and the four steps
-// of A v, dealt to the waves in turn) meet in shared memory once a chunk and are added in the order of the
-// waves.  The shares of o that the token-by-token kernel would leave in further planes of `out` are zero here.
+// A wave's chain per chunk is nine matrix instructions; the waves' shares of the chunks' o (and the four steps
+// of A v, dealt to the waves in turn) meet in shared memory, a barrier every few chunks, and are added in the
+// order of the waves.  The shares of o that the token-by-token kernel would leave in further planes of `out` are zero here.
 template <typename T, int NW>
 __global__ __launch_bounds__(64 * NW) void gla_chunk_scan_kernel(
     const T* __restrict__ proj, int64_t proj_stride, int v_off, const float* __restrict__ work,
     float* __restrict__ state, const int32_t* __restrict__ q_starts, const int32_t* __restrict__ seq_slots,
     float* __restrict__ out, int64_t out_plane, int heads, int dim, int vdim, int dp, int planes, int n_slots) {
-    __shared__ float part[2][NW][4][64];
+    constexpr int G = NW <= 8 ? 4 : 2;  // chunks between two barriers: their shares of o lie in LDS side by side
+    __shared__ float part[2][G][NW][4][64];
     const int seq = blockIdx.x, h = blockIdx.y;
     const int n_chunks = gla_chunks_of(q_starts, seq_slots, seq, n_slots);
     if (n_chunks == 0) return;  // the same for the whole workgroup
@@ -336,20 +337,20 @@ __global__ __launch_bounds__(64 * NW) void gla_chunk_scan_kernel(
         g4v[slot_] = *reinterpret_cast<const floatx4*>(wc + g_at);
         a4[slot_] = *reinterpret_cast<const floatx4*>(wc + a_at);
     };
-    // o of chunk ci from the waves' shares, added in the order of the waves (the first 256 threads, one value
-    // each; with fewer threads, several).  Further planes of `out`: zeros.
-    auto finish = [&](int ci, bool really) {
-        const int t0 = lo + ci * kGlaChunk;
+    // o of the `count` chunks of group gi (G chunks between two barriers) from the waves' shares, added in the
+    // order of the waves, a value a thread and round.  Further planes of `out`: zeros.
+    auto finish = [&](int gi, int count, bool really) {
+        const int t0 = lo + gi * G * kGlaChunk;
         float* oc = out + static_cast<int64_t>(t0) * out_stride + h * vdim + blockIdx.z * 16;
 #pragma unroll
-        for (int e0 = 0; e0 < 256; e0 += 64 * NW) {
+        for (int e0 = 0; e0 < 256 * G; e0 += 64 * NW) {
             const int e = e0 + tid;
-            if (e < 256) {
-                const int i = e >> 6, l = e & 63;
-                float sum = part[ci & 1][0][i][l];
+            const int j = e >> 8, i = (e >> 6) & 3, l = e & 63;
+            if (j < count) {
+                float sum = part[gi & 1][j][0][i][l];
 #pragma unroll
-                for (int ww = 1; ww < NW; ++ww) sum += part[ci & 1][ww][i][l];
-                const int tok = 4 * (l >> 4) + i, c = l & 15;
+                for (int ww = 1; ww < NW; ++ww) sum += part[gi & 1][j][ww][i][l];
+                const int tok = j * kGlaChunk + 4 * (l >> 4) + i, c = l & 15;
                 if (really && t0 + tok < hi && blockIdx.z * 16 + c < vdim) {
                     float* dst = oc + tok * static_cast<int>(out_stride) + c;
                     *dst = sum;
@@ -381,18 +382,20 @@ __global__ __launch_bounds__(64 * NW) void gla_chunk_scan_kernel(
                 S *= g4v[u];
 #pragma unroll
                 for (int m = 0; m < 4; ++m) S = __builtin_amdgcn_mfma_f32_16x16x4f32(k4[u][m], v[u][m], S, 0, 0, 0);
-                // the chunk before this one: its shares lie in the other half of `part` since the last barrier;
+                // the group before this one: its shares lie in the other half of `part` since the last barrier;
                 // adding them up and storing o goes on while the matrix instructions above are at work
-                finish(ci - 1, ci > 0);
+                const int gi = ci / G;
+                if (u % G == 0) finish(gi - 1, G, gi > 0);
                 const floatx4 mine = o[0] + o[1];
 #pragma unroll
-                for (int i = 0; i < 4; ++i) part[ci & 1][wave][i][lane] = mine[i];
-                // everyone has written this chunk's half and has read the other: the next chunk may overwrite that
-                lds_barrier();
+                for (int i = 0; i < 4; ++i) part[gi & 1][u % G][wave][i][lane] = mine[i];
+                // at a group's end everyone has written its half and has read the other: the next group may
+                // overwrite that
+                if (u % G == G - 1 || ci == n_chunks - 1) lds_barrier();
             }
         }
     }
-    finish(n_chunks - 1, true);
+    finish((n_chunks - 1) / G, n_chunks - (n_chunks - 1) / G * G, true);
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         const int row = ch0 + 4 * g4 + i;
