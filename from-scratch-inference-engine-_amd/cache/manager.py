@@ -126,6 +126,12 @@ class CacheManager:
             return 0
         return max(0, length - window + 1) // self.tokens_per_page(group)
 
+    def kept_pages(self, group: int) -> int:
+        """Pages at a request's start that a windowed group never hands back: they hold the first positions that
+        the group's need says every query keeps reading."""
+        keep = int(getattr(self.groups[group], "keep_first", 0) or 0)
+        return self.pages_for(keep, group) if keep > 0 else 0
+
     def new_pages_needed(self, rc: RequestCache, n_tokens: int) -> List[int]:
         """Pages each group must take from its pool to hold ``n_tokens`` more."""
         return [max(0, self.pages_for(rc.length + n_tokens, g) - len(t)) for g, t in enumerate(rc.tables)]
@@ -139,7 +145,7 @@ class CacheManager:
                 out.append(self.pages_for(total_tokens, g))
             else:
                 span = min(total_tokens, need.window + portion + self.tokens_per_page(g))
-                out.append(min(self.pages_for(total_tokens, g), self.pages_for(span, g) + 1))
+                out.append(min(self.pages_for(total_tokens, g), self.pages_for(span, g) + 1 + self.kept_pages(g)))
         return out
 
     def can_reserve(self, items: Iterable[Tuple[RequestCache, int]]) -> bool:
@@ -182,7 +188,7 @@ class CacheManager:
             if self.groups[g].window is None:
                 continue
             dead = min(self.first_needed_page(g, rc.length), len(table))
-            for idx in range(dead):
+            for idx in range(min(self.kept_pages(g), dead), dead):
                 if table[idx] >= 0:
                     self.allocators[g].free(table[idx])
                     table[idx] = -1

@@ -46,6 +46,7 @@ from typing import Optional, Tuple
 class CacheNeed:
     per_token: bool = True
     window: Optional[int] = None
+    keep_first: int = 0  # positions at a request's start whose pages a window never hands back
     # Per-token needs: how the positions of a request map to the entries of its pages.  One entry
     # holds ``tokens_per_entry`` consecutive positions (1: an entry a token; k: a mixer that keeps
     # one record per block of k tokens), and a page of this need's group has ``page_entries``
@@ -101,6 +102,8 @@ class PagedNeed(CacheNeed):
     n_kv_heads: int
     head_dim: int
     window: Optional[int] = None
+    # with a window: the first positions of a request that every later query still reads (their pages stay)
+    keep_first: int = 0
     per_token = True
 
     def __post_init__(self):
@@ -108,6 +111,8 @@ class PagedNeed(CacheNeed):
             raise ValueError("PagedNeed: sizes must be positive")
         if self.window is not None and self.window < 1:
             raise ValueError("PagedNeed: window must be >= 1")
+        if self.keep_first < 0:
+            raise ValueError("PagedNeed: keep_first must be >= 0")
 
     def allocate(self, n_caches, units, page_size, device, dtype):
         import torch

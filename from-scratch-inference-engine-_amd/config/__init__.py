@@ -1,7 +1,8 @@
 """Typed model configurations read from config.json."""
 
 from .base import ConfigError, ModelConfig, read_config_json
+from .botulorn import BotulornConfig
 from .gilozen import GilozenConfig
 from .qwen2 import Qwen2Config
 
-__all__ = ["ConfigError", "GilozenConfig", "ModelConfig", "Qwen2Config", "read_config_json"]
+__all__ = ["BotulornConfig", "ConfigError", "GilozenConfig", "ModelConfig", "Qwen2Config", "read_config_json"]

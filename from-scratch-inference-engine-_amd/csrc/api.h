@@ -24,6 +24,10 @@
 #define FSIE_ATTN_ITEM_KBEGIN 4   // first key
 #define FSIE_ATTN_ITEM_KEND 5     // one past the last key
 #define FSIE_ATTN_ITEM_PARTIAL 6  // -1: write the output; >= 0: first partial slot of the tile
+// The first tokens of a request that a window keeps: keys below KEEP are seen whatever the window says.  With
+// FSIE_ATTN_KEEP_WALK set the item also reads the keys [0, min(KEEP, KBEGIN)), before those of its own range.
+#define FSIE_ATTN_ITEM_KEEP 7
+#define FSIE_ATTN_KEEP_WALK (1 << 30)
 // one merge item = 4 int32: {output row, first partial slot, number of splits, slot stride}
 #define FSIE_ATTN_MERGE_INTS 4
 
@@ -80,6 +84,7 @@ int fsie_gla_scan(const void* proj, int64_t proj_stride, int q_off, int k_off, i
 
 // Attention through a latent (latent_attention.hip): the norms of the latents, the gates and the cache row of
 // every token; the rotation of pairs of neighbours; a product with a matrix of its own for every head.
+// rot_pairs > 0: the rotated pairs are neighbours (2i, 2i + 1); rot_pairs < 0: -rot_pairs pairs (i, i + pairs)
 int fsie_latent_prep(const void* proj, int64_t stride, int dq_off, int q_rank, int dkv_off, int kv_rank, int rot_dim,
                      int rot_pairs, int g_off, int heads, const float* q_weight, const float* kv_weight, float eps,
                      const float* cos_sin, void* cq, float* gate, const int32_t* slots, void* k_pool, void* v_pool,
@@ -105,6 +110,32 @@ int fsie_rope_kv_write_table(void* qkv, const float* cos_sin, const int32_t* slo
 
 // table [n_tokens, half, 2] float32: cos and sin of positions[t] * inv_freq[i]
 int fsie_rope_table(const int32_t* positions, const double* inv_freq, int n_tokens, int half, float* table,
+                    hipStream_t stream);
+
+// the same with every cosine and sine multiplied by `magnitude` (rotations whose scaling of the frequencies
+// comes with a factor on the rotated vectors)
+int fsie_rope_table_scaled(const int32_t* positions, const double* inv_freq, int n_tokens, int half, float magnitude,
+                           float* table, hipStream_t stream);
+
+// Layer norm over the residual stream, fused with the residual sum of up to two pending deltas (parts: 0 = one
+// array of the activations' type, n = n float32 partial sums), one or two outputs that differ in weight and bias.
+int fsie_layer_norm(float* residual, const void* delta_a, int parts_a, const void* delta_b, int parts_b, const float* w1,
+                    const float* b1, void* out1, const float* w2, const float* b2, void* out2, const int32_t* rows,
+                    int n_rows, int hidden, float eps, int dtype, int write_back, int total_rows, hipStream_t stream);
+// Token rows times `scale` plus the hashed row of (previous token, token); last[slot] keeps a request's latest
+// token + 1 from step to step (0: none) and is brought up to date after the rows are written.
+int fsie_pair_embedding(const void* table, const void* pairs, int dtype, const int32_t* ids, const int32_t* q_starts,
+                        const int32_t* seq_slots, int n_seqs, int32_t* last, int n_slots, float* out, int n_tokens,
+                        int hidden, int vocab, int buckets, int64_t mul_prev, int64_t mul_cur, float scale,
+                        hipStream_t stream);
+// Between the fused q|k|v|gate projection and attention: head norms, partial rotation from the step's table, the
+// mixing of values with another layer's, the gates' sigmoid, queries and cache entries in heads of D values.
+int fsie_attention_prep(const void* proj, int64_t stride, int q_off, int k_off, int v_off, int g_off, int heads,
+                        int kv_heads, int dim, int vdim, int D, const float* q_weight, const float* k_weight, float eps,
+                        int pairs, const float* cos_sin, const void* v_other, int64_t v_other_stride, const float* mix,
+                        void* q_out, float* gate, const int32_t* slots, void* k_pool, void* v_pool, int page_size,
+                        int64_t pool_slots, int n_tokens, int dtype, hipStream_t stream);
+int fsie_gate_heads(const void* x, int D, const float* gate, void* y, int n_tokens, int heads, int vdim, int dtype,
                     hipStream_t stream);
 
 int fsie_gemm(const void* x, const void* w, const float* bias, void* y, int M, int N, int K, int dtype,

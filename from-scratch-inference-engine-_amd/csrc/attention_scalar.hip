@@ -69,6 +69,10 @@ __global__ __launch_bounds__(256) void attention_scalar_kernel(
     const int key_end = item[FSIE_ATTN_ITEM_KEND];
     const int partial_base = item[FSIE_ATTN_ITEM_PARTIAL];
     if (n_q <= 0) return;  // padding item
+    // the first keys that a window keeps: seen whatever the window says, and read before the item's own
+    // range where the item is told to
+    const int keep = item[FSIE_ATTN_ITEM_KEEP] & ~FSIE_ATTN_KEEP_WALK;
+    const int prefix_end = (item[FSIE_ATTN_ITEM_KEEP] & FSIE_ATTN_KEEP_WALK) ? min(keep, key_begin) : 0;
 
     const int group = n_heads / n_kv;
     const int kvh = blockIdx.y / head_chunks;
@@ -105,8 +109,10 @@ __global__ __launch_bounds__(256) void attention_scalar_kernel(
     const int n_chunks = (hd + 31) / 32;
     const int32_t* table = block_tables + static_cast<int64_t>(seq) * max_pages;
 
-    const bool slots_by_four = VEC && (key_begin & 3) == 0;
-    for (int kt = key_begin; kt < key_end; kt += kKeys) {
+    for (int seg = prefix_end > 0 ? 0 : 1; seg < 2; ++seg) {
+    const int seg_begin = seg ? key_begin : 0, seg_end = seg ? key_end : prefix_end;
+    const bool slots_by_four = VEC && (seg_begin & 3) == 0;
+    for (int kt = seg_begin; kt < seg_end; kt += kKeys) {
         __syncthreads();  // previous tile's values are no longer read (first pass: qs is written)
         if (VEC) {
             const int per_key = hd >> 2;
@@ -114,7 +120,7 @@ __global__ __launch_bounds__(256) void attention_scalar_kernel(
                 const int j = e / per_key, d = (e - j * per_key) * 4;
                 const int kj = kt + j;
                 float f[4] = {0.f, 0.f, 0.f, 0.f};
-                if (kj < key_end) {
+                if (kj < seg_end) {
                     const int page = table[kj / page_size];
                     if (page >= 0)
                         load4(k_pool + ((static_cast<int64_t>(page) * n_kv + kvh) * page_size + kj % page_size) * hd + d, f);
@@ -127,7 +133,7 @@ __global__ __launch_bounds__(256) void attention_scalar_kernel(
                 const int j = e / hd, d = e - j * hd;
                 const int kj = kt + j;
                 float v = 0.f;
-                if (kj < key_end) {
+                if (kj < seg_end) {
                     const int page = table[kj / page_size];
                     if (page >= 0) {
                         v = to_float(k_pool[((static_cast<int64_t>(page) * n_kv + kvh) * page_size + kj % page_size) * hd + d]);
@@ -144,7 +150,7 @@ __global__ __launch_bounds__(256) void attention_scalar_kernel(
             const bool row_ok = r < n_rows && (r % gh) < gh_here;
             const int pos = pos0 + r / gh;
             const int kj = kt + lane32;
-            bool visible = row_ok && kj < key_end && kj <= pos && (window <= 0 || kj > pos - window);
+            bool visible = row_ok && kj < seg_end && kj <= pos && (window <= 0 || kj > pos - window || kj < keep);
             if (visible) visible = table[kj / page_size] >= 0;
             float s = -INFINITY;
             if (visible) {
@@ -169,20 +175,20 @@ __global__ __launch_bounds__(256) void attention_scalar_kernel(
                 const int g = e & (kKeys / 4 - 1), d = e / (kKeys / 4);
                 const int kj = kt + 4 * g;  // a multiple of 4: the four slots lie in one page
                 float f[4] = {0.f, 0.f, 0.f, 0.f};
-                if (kj < key_end) {
+                if (kj < seg_end) {
                     const int page = table[kj / page_size];
                     if (page >= 0)
                         load4(v_pool + ((static_cast<int64_t>(page) * n_kv + kvh) * hd + d) * page_size + kj % page_size, f);
                 }
 #pragma unroll
-                for (int t = 0; t < 4; ++t) kv[(4 * g + t) * kv_stride + d] = kj + t < key_end ? f[t] : 0.f;
+                for (int t = 0; t < 4; ++t) kv[(4 * g + t) * kv_stride + d] = kj + t < seg_end ? f[t] : 0.f;
             }
         } else {
             for (int e = tid; e < kKeys * hd; e += blockDim.x) {
                 const int j = e / hd, d = e - j * hd;
                 const int kj = kt + j;
                 float v = 0.f;
-                if (kj < key_end) {
+                if (kj < seg_end) {
                     const int page = table[kj / page_size];
                     if (page >= 0) {
                         v = to_float(v_pool[((static_cast<int64_t>(page) * n_kv + kvh) * hd + d) * page_size + kj % page_size]);
@@ -208,6 +214,7 @@ __global__ __launch_bounds__(256) void attention_scalar_kernel(
                 }
             }
         }
+    }
     }
 
     // results

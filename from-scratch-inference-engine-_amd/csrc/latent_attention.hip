@@ -17,12 +17,20 @@ namespace {
 
 constexpr int kThreads = 256;
 
-// Element j of a run of `width` values of which the first 2 * pairs are pairs (2i, 2i + 1) turned by
-// the angles whose cosines and sines are cs[i]; the rest passes.
+// Element j of a run of `width` values of which the first 2 * |pairs| are turned by the angles whose cosines
+// and sines are cs[i]; the rest passes.  pairs > 0: the pairs are neighbours (2i, 2i + 1); pairs < 0: value i
+// goes with value i + |pairs|.
 template <typename T>
 __device__ __forceinline__ float rotated_neighbour(const T* __restrict__ run, int j, int pairs, const float2* __restrict__ cs) {
     const float x = to_float(run[j]);
-    if (j >= 2 * pairs) return x;
+    const int n = pairs < 0 ? -pairs : pairs;
+    if (j >= 2 * n) return x;
+    if (pairs < 0) {
+        const bool low = j < n;
+        const float2 t = cs[low ? j : j - n];
+        const float other = to_float(run[low ? j + n : j - n]);
+        return low ? fmaf(x, t.x, -(other * t.y)) : fmaf(x, t.x, other * t.y);
+    }
     const float2 t = cs[j >> 1];
     const float other = to_float(run[j ^ 1]);
     return (j & 1) ? fmaf(x, t.x, other * t.y) : fmaf(x, t.x, -(other * t.y));
@@ -63,7 +71,7 @@ __global__ __launch_bounds__(kThreads) void latent_prep_kernel(
     if (slot < 0 || slot >= pool_slots) return;
     const int64_t page = slot / page_size;
     const int off = static_cast<int>(slot - page * page_size);
-    const float2* cs = cos_sin + static_cast<int64_t>(t) * pairs;
+    const float2* cs = cos_sin + static_cast<int64_t>(t) * (pairs < 0 ? -pairs : pairs);
     for (int j = threadIdx.x; j < width; j += kThreads) {
         float v = 0.f;
         if (j < kv_rank) v = (to_float(x[j]) * scale) * kv_weight[j];
@@ -82,7 +90,7 @@ __global__ __launch_bounds__(kThreads) void rope_pairs_kernel(const T* __restric
                                                               int heads, int width, int pairs, int out_width,
                                                               const float2* __restrict__ cos_sin) {
     const int t = blockIdx.x;
-    const float2* cs = cos_sin + static_cast<int64_t>(t) * pairs;
+    const float2* cs = cos_sin + static_cast<int64_t>(t) * (pairs < 0 ? -pairs : pairs);
     for (int e = threadIdx.x; e < heads * out_width; e += kThreads) {
         const int h = e / out_width, j = e - h * out_width;
         const float v = j < width ? rotated_neighbour(in + static_cast<int64_t>(t) * in_stride + in_off + h * in_hs, j, pairs, cs) : 0.f;
@@ -229,9 +237,9 @@ extern "C" int fsie_latent_prep(const void* proj, int64_t stride, int dq_off, in
                                 const int32_t* slots, void* k_pool, void* v_pool, int width, int page_size,
                                 int64_t pool_slots, int n_tokens, int dtype, hipStream_t stream) {
     FSIE_REQUIRE(n_tokens >= 0 && q_rank > 0 && kv_rank > 0 && rot_dim >= 0 && heads >= 0, "latent_prep: bad sizes");
-    FSIE_REQUIRE(rot_pairs >= 0 && 2 * rot_pairs <= rot_dim, "latent_prep: %d rotated pairs do not fit %d values", rot_pairs, rot_dim);
+    FSIE_REQUIRE(2 * abs(rot_pairs) <= rot_dim, "latent_prep: %d rotated pairs do not fit %d values", rot_pairs, rot_dim);
     FSIE_REQUIRE(dtype == FSIE_F32 || dtype == FSIE_BF16, "latent_prep: unknown dtype %d", dtype);
-    FSIE_REQUIRE(proj && q_weight && cq && gate, "latent_prep: missing operand");
+    FSIE_REQUIRE(proj && q_weight && cq && (gate || heads == 0), "latent_prep: missing operand");
     FSIE_REQUIRE(dq_off >= 0 && dq_off + q_rank <= stride && g_off >= 0 && g_off + heads <= stride,
                  "latent_prep: the columns do not fit a row of %lld", static_cast<long long>(stride));
     const bool writes = k_pool != nullptr;
@@ -257,7 +265,7 @@ extern "C" int fsie_latent_prep(const void* proj, int64_t stride, int dq_off, in
 extern "C" int fsie_rope_pairs(const void* in, int64_t in_stride, int in_off, int in_hs, void* out, int64_t out_stride,
                                int out_off, int out_hs, int heads, int width, int rot_pairs, int out_width,
                                const float* cos_sin, int n_tokens, int dtype, hipStream_t stream) {
-    FSIE_REQUIRE(n_tokens >= 0 && heads > 0 && width >= 0 && out_width >= width && 2 * rot_pairs <= width && rot_pairs >= 0,
+    FSIE_REQUIRE(n_tokens >= 0 && heads > 0 && width >= 0 && out_width >= width && 2 * abs(rot_pairs) <= width,
                  "rope_pairs: bad sizes heads=%d width=%d pairs=%d out_width=%d", heads, width, rot_pairs, out_width);
     FSIE_REQUIRE(dtype == FSIE_F32 || dtype == FSIE_BF16, "rope_pairs: unknown dtype %d", dtype);
     FSIE_REQUIRE(in && out && (rot_pairs == 0 || cos_sin) && reinterpret_cast<uintptr_t>(cos_sin) % 8 == 0, "rope_pairs: missing operand");

@@ -48,6 +48,9 @@ def _require_gpu(device) -> torch.device:
     return device
 
 
+EMBEDDING_CACHE = -1  # the cache id of what the embedding keeps (the schedule's calls count from 0)
+
+
 class Model:
     def __init__(self, spec: ModelSpec, dtype, device):
         self.spec = spec
@@ -70,6 +73,12 @@ class Model:
                 if not 0 <= call.cache_of < i or spec.schedule[call.cache_of].cache_of is not None:
                     raise ValueError(f"schedule entry {i}: cache_of must name an earlier call that keeps a cache")
                 self.call_cache.append(call.cache_of)
+        # what the embedding keeps for a request between steps (a per-request need), under an id of its own
+        embedding_need = spec.embedding.cache_need()
+        if embedding_need is not None:
+            if getattr(embedding_need, "per_token", True):
+                raise TypeError("the embedding's cache need must be a per-request one")
+            needs[EMBEDDING_CACHE] = embedding_need
         # per-token needs that compare equal share a pool of pages (a group); a per-request need
         # gets slots of its own.  What the memory looks like is the need's business.
         groups: List[CacheNeed] = []
@@ -181,7 +190,8 @@ class Model:
         ctx.memo.clear()  # a captured graph must hold whatever the layers share: nothing is kept from an earlier pass
         storage.reset_states(ctx)  # requests that start in this step find their per-request memory zero
         storage.clear_fresh(ctx)   # and the pages taken from the pools for this step hold nothing of their last owner
-        hidden = HiddenState(spec.embedding.forward(ctx.token_ids))
+        kept = storage.view(EMBEDDING_CACHE, ctx, writes=True) if EMBEDDING_CACHE in self.cached_calls else None
+        hidden = HiddenState(spec.embedding.embed(ctx, kept))
         for i, call in enumerate(spec.schedule):
             cid = self.call_cache[i]
             cache = storage.view(cid, ctx, writes=call.cache_of is None) if cid in self.cached_calls else None

@@ -64,6 +64,12 @@ def bind(bindings: List[ParamBinding], owner: Part, attr: str, sources: Sequence
     """Declare that ``owner.attr`` is made of the checkpoint tensors ``sources`` (joined along
     dim 0 the way the part's declaration says); checks the shapes against that declaration."""
     decl = owner.param_decls()[attr]
+    if tuple(decl.shape) == ():
+        # a single number: one checkpoint tensor without dimensions
+        if len(sources) != 1 or tuple(sources[0].shape) != ():
+            raise ValueError(f"{type(owner).__name__}.{attr}: a single number is one tensor of shape ()")
+        bindings.append(ParamBinding(owner, attr, list(sources), decl.storage, decl.layout))
+        return
     rows = sum(s.shape[0] for s in sources)
     tail = tuple(sources[0].shape[1:])
     if any(tuple(s.shape[1:]) != tail for s in sources) or (rows, *tail) != tuple(decl.shape):

@@ -12,7 +12,8 @@ from .functions import (FragmentOrdered, attention_merge, attention_mfma, attent
                         gemm_mfma_wide_swiglu, gemm_mfma_wide_takes, random_fill,
                         residual_add,
                         rmsnorm, rmsnorm_plain, rope_kv_write, rope_table, sample, swiglu, zero_pages, zero_rows,
-                        gate_act_code, gated_headnorm, gla_scan, head_gemm, latent_prep, rope_pairs, sandwich_norm, softcap)
+                        gate_act_code, gated_headnorm, gla_scan, head_gemm, latent_prep, rope_pairs, sandwich_norm, softcap,
+                        attention_prep, gate_heads, layer_norm, pair_embedding)
 from .library import KernelError, KernelLibraryMissing, load
 from .tuning import disable_library_tuning, enable_library_tuning, library_mm, library_tuning_enabled
 
@@ -22,4 +23,5 @@ __all__ = ["FragmentOrdered", "KernelError", "KernelLibraryMissing", "attention_
            "enable_library_tuning", "fragment_order", "gemm", "gemm_mfma_fp32", "gemm_mfma_skinny", "gemm_mfma_skinny_rope", "gemm_mfma_wide",
            "gemm_mfma_wide_best_splits", "gemm_mfma_wide_splits_ok", "gemm_mfma_wide_swiglu", "gemm_mfma_wide_takes", "library_mm", "library_tuning_enabled", "load", "random_fill", "residual_add",
            "rmsnorm", "rmsnorm_plain", "rope_kv_write", "rope_table", "sample", "swiglu", "zero_pages", "zero_rows",
-           "gate_act_code", "gated_headnorm", "gla_scan", "head_gemm", "latent_prep", "rope_pairs", "sandwich_norm", "softcap"]
+           "gate_act_code", "gated_headnorm", "gla_scan", "head_gemm", "latent_prep", "rope_pairs", "sandwich_norm", "softcap",
+           "attention_prep", "gate_heads", "layer_norm", "pair_embedding"]

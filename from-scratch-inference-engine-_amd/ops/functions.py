@@ -13,6 +13,7 @@ from .library import KernelError, check, load
 F32, BF16 = 0, 1
 ATTN_ITEM_INTS = 8
 ATTN_MERGE_INTS = 4
+ATTN_KEEP_WALK = 1 << 30  # in an item's last field, beside the number of kept first keys: read them before the item's range
 GEMM_SKINNY_MAX_M = 8
 GEMM_MFMA_SKINNY_MAX_M = 64
 GEMM_MFMA_WIDE_MAX_M = 128  # the product that shares x through LDS, on a fragment-ordered weight
@@ -491,15 +492,16 @@ def gemm_mfma_skinny_rope(x: torch.Tensor, weight: torch.Tensor, bias: Optional[
     return out
 
 
-def rope_table(positions: torch.Tensor, inv_freq: torch.Tensor) -> torch.Tensor:
+def rope_table(positions: torch.Tensor, inv_freq: torch.Tensor, magnitude: float = 1.0) -> torch.Tensor:
     """float32 [T, half, 2]: cos and sin of positions[t] * inv_freq[i] (the angle in float64, as in
-    the kernels that rotate).  The angles of a step are the same in every layer: a step makes the
-    table once."""
+    the kernels that rotate), each times ``magnitude``.  The angles of a step are the same in every
+    layer: a step makes the table once."""
     _need(positions, "positions", dtype=torch.int32, ndim=1)
     _need(inv_freq, "inv_freq", dtype=torch.float64, ndim=1)
     t, half = positions.shape[0], inv_freq.shape[0]
     table = torch.empty((t, half, 2), dtype=torch.float32, device=positions.device)
-    check(load().fsie_rope_table(positions.data_ptr(), inv_freq.data_ptr(), t, half, table.data_ptr(), _stream()))
+    check(load().fsie_rope_table_scaled(positions.data_ptr(), inv_freq.data_ptr(), t, half, float(magnitude),
+                                        table.data_ptr(), _stream()))
     return table
 
 
@@ -829,7 +831,8 @@ def latent_prep(proj: torch.Tensor, dq_off: int, q_rank: int, dkv_off: int, kv_r
                 k_pool: Optional[torch.Tensor] = None, v_pool: Optional[torch.Tensor] = None):
     """From the fused projection ``proj`` [T, W]: the normed query latent [T, q_rank] (type of ``proj``), the
     sigmoid of the heads' gates (float32 [T, heads]) and, if pools are given, every token's cache row
-    [normed latent | key part with its first ``rot_pairs`` pairs of neighbours rotated | zeros] written at
+    [normed latent | key part with its first ``rot_pairs`` pairs of neighbours rotated (a negative number: that
+    many pairs of value i with value i + pairs) | zeros] written at
     ``slots`` into ``k_pool`` [units, 1, page, width] and (transposed) ``v_pool`` [units, 1, width, page]."""
     _need(proj, "latent proj", ndim=2)
     t, w = proj.shape
@@ -845,7 +848,7 @@ def latent_prep(proj: torch.Tensor, dq_off: int, q_rank: int, dkv_off: int, kv_r
         _need(kv_weight, "latent kv norm weight", dtype=torch.float32, shape=(kv_rank,))
         pool_slots = units * page_size
         if rot_pairs:
-            _need(cos_sin, "latent cos/sin", dtype=torch.float32, shape=(t, rot_pairs, 2))
+            _need(cos_sin, "latent cos/sin", dtype=torch.float32, shape=(t, abs(rot_pairs), 2))
     cq = torch.empty((t, q_rank), dtype=proj.dtype, device=proj.device)
     gate = torch.empty((t, heads), dtype=torch.float32, device=proj.device)
     check(load().fsie_latent_prep(proj.data_ptr(), w, dq_off, q_rank, dkv_off, kv_rank, rot_dim, rot_pairs, g_off, heads,
@@ -858,7 +861,8 @@ def latent_prep(proj: torch.Tensor, dq_off: int, q_rank: int, dkv_off: int, kv_r
 def rope_pairs(x: torch.Tensor, in_off: int, in_head_stride: int, out: torch.Tensor, out_off: int, out_head_stride: int,
                heads: int, width: int, rot_pairs: int, out_width: int, cos_sin: Optional[torch.Tensor]) -> torch.Tensor:
     """Of every token and head the run of ``width`` values at column ``in_off + h * in_head_stride`` of ``x``,
-    its first ``rot_pairs`` pairs of neighbours (2i, 2i + 1) rotated by ``cos_sin`` [T, rot_pairs, 2], written to
+    its first ``rot_pairs`` pairs of neighbours (2i, 2i + 1) rotated by ``cos_sin`` [T, rot_pairs, 2] (a negative
+    ``rot_pairs``: that many pairs of value i with value i + pairs), written to
     column ``out_off + h * out_head_stride`` of ``out`` and filled up with zeros to ``out_width`` values."""
     _need(x, "rope_pairs x", ndim=2)
     _need(out, "rope_pairs out", dtype=x.dtype, ndim=2)
@@ -866,7 +870,7 @@ def rope_pairs(x: torch.Tensor, in_off: int, in_head_stride: int, out: torch.Ten
     if out.shape[0] != t:
         raise KernelError("rope_pairs: x and out must have a row a token")
     if rot_pairs:
-        _need(cos_sin, "rope_pairs cos/sin", dtype=torch.float32, shape=(t, rot_pairs, 2))
+        _need(cos_sin, "rope_pairs cos/sin", dtype=torch.float32, shape=(t, abs(rot_pairs), 2))
     check(load().fsie_rope_pairs(x.data_ptr(), x.shape[1], in_off, in_head_stride, out.data_ptr(), out.shape[1], out_off,
                                  out_head_stride, heads, width, rot_pairs, out_width, _ptr(cos_sin), t,
                                  dtype_code(x.dtype), _stream()))
@@ -891,3 +895,128 @@ def head_gemm(x: torch.Tensor, x_off: int, x_head_stride: int, weight: torch.Ten
                                 out.shape[1], out_off, out_head_stride, _ptr(gate), t, heads, n, k, dtype_code(x.dtype),
                                 _stream()))
     return out
+
+
+def _delta_parts(delta: Optional[torch.Tensor], t: int, h: int, out_dtype: torch.dtype, name: str) -> int:
+    """How a pending delta comes: 0 = one array [T, H] of the activations' type, n = float32 partial sums [n, T, H]."""
+    if delta is None:
+        return 0
+    if delta.ndim == 3:
+        n = delta.shape[0]
+        _need(delta, f"{name} delta parts", dtype=torch.float32, shape=(n, t, h))
+        if not 1 <= n <= GEMM_MAX_SPLITS:
+            raise KernelError(f"{name}: {n} partial sums; up to {GEMM_MAX_SPLITS} are taken")
+        return n
+    _need(delta, f"{name} delta", dtype=out_dtype, shape=(t, h))
+    return 0
+
+
+def layer_norm(residual: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor, eps: float, out_dtype: torch.dtype,
+               delta: Optional[torch.Tensor] = None, delta2: Optional[torch.Tensor] = None,
+               weight2: Optional[torch.Tensor] = None, bias2: Optional[torch.Tensor] = None,
+               rows: Optional[torch.Tensor] = None, write_back: bool = False):
+    """Layer norm of ``residual + delta + delta2`` (float32 stream; each delta [T, H] in ``out_dtype`` or float32
+    partial sums [S, T, H] added in order), ``(v - mean) / sqrt(var + eps) * weight + bias`` with the variance the
+    mean of the squared deviations, all in float32.  With ``weight2`` and ``bias2`` a second output from the same
+    statistics: the function then returns both.  ``write_back`` stores the sum into ``residual``; ``rows`` (int32)
+    selects rows."""
+    _need(residual, "layer_norm residual", dtype=torch.float32, ndim=2)
+    t, h = residual.shape
+    _need(weight, "layer_norm weight", dtype=torch.float32, shape=(h,))
+    _need(bias, "layer_norm bias", dtype=torch.float32, shape=(h,))
+    two = weight2 is not None
+    if two:
+        _need(weight2, "layer_norm second weight", dtype=torch.float32, shape=(h,))
+        _need(bias2, "layer_norm second bias", dtype=torch.float32, shape=(h,))
+    parts_a = _delta_parts(delta, t, h, out_dtype, "layer_norm")
+    parts_b = _delta_parts(delta2, t, h, out_dtype, "layer_norm")
+    n_rows = t
+    if rows is not None:
+        _need(rows, "layer_norm rows", dtype=torch.int32, ndim=1)
+        n_rows = rows.shape[0]
+    out = torch.empty((n_rows, h), dtype=out_dtype, device=residual.device)
+    out2 = torch.empty((n_rows, h), dtype=out_dtype, device=residual.device) if two else None
+    check(load().fsie_layer_norm(residual.data_ptr(), _ptr(delta), parts_a, _ptr(delta2), parts_b, weight.data_ptr(),
+                                 bias.data_ptr(), out.data_ptr(), _ptr(weight2), _ptr(bias2), _ptr(out2), _ptr(rows), n_rows,
+                                 h, float(eps), dtype_code(out_dtype), int(write_back), t, _stream()))
+    return (out, out2) if two else out
+
+
+def pair_embedding(table: torch.Tensor, pairs: torch.Tensor, ids: torch.Tensor, q_starts: torch.Tensor,
+                   seq_slots: torch.Tensor, last: torch.Tensor, mul_prev: int, mul_cur: int, scale: float) -> torch.Tensor:
+    """float32 rows ``table[id] * scale + pairs[(previous id * mul_prev + id * mul_cur) mod buckets]`` with
+    ``buckets = pairs.shape[0] - 1``; a request's first token takes the last row of ``pairs``.  ``q_starts`` int32
+    [requests + 1] and ``seq_slots`` int32 [requests] describe the step; ``last`` int32 [slots, 1] keeps every
+    request's latest id + 1 between steps (0: none yet) and is brought up to date."""
+    _need(table, "pair_embedding table", ndim=2)
+    _need(pairs, "pair_embedding pairs", dtype=table.dtype, ndim=2)
+    _need(ids, "pair_embedding ids", dtype=torch.int32, ndim=1)
+    _need(q_starts, "pair_embedding q_starts", dtype=torch.int32, ndim=1)
+    _need(seq_slots, "pair_embedding seq_slots", dtype=torch.int32, shape=(q_starts.shape[0] - 1,))
+    _need(last, "pair_embedding last tokens", dtype=torch.int32)
+    v, h = table.shape
+    if pairs.shape[1] != h or pairs.shape[0] < 2:
+        raise KernelError(f"pair_embedding: the pairs' table {tuple(pairs.shape)} does not go with rows of {h}")
+    t = ids.shape[0]
+    out = torch.empty((t, h), dtype=torch.float32, device=table.device)
+    check(load().fsie_pair_embedding(table.data_ptr(), pairs.data_ptr(), dtype_code(table.dtype), ids.data_ptr(),
+                                     q_starts.data_ptr(), seq_slots.data_ptr(), seq_slots.shape[0], last.data_ptr(),
+                                     last.numel(), out.data_ptr(), t, h, v, pairs.shape[0] - 1, int(mul_prev), int(mul_cur),
+                                     float(scale), _stream()))
+    return out
+
+
+def attention_prep(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, g_off: int, heads: int, kv_heads: int, dim: int,
+                   vdim: int, padded: int, q_weight: Optional[torch.Tensor], k_weight: Optional[torch.Tensor], eps: float,
+                   pairs: int, cos_sin: Optional[torch.Tensor], gated: bool, v_other: Optional[torch.Tensor] = None,
+                   v_other_stride: int = 0, mix: Optional[torch.Tensor] = None, slots: Optional[torch.Tensor] = None,
+                   k_pool: Optional[torch.Tensor] = None, v_pool: Optional[torch.Tensor] = None):
+    """From the fused projection ``proj`` [T, W] (q, k, v and one gate logit a head at their column offsets): the
+    queries [T, heads * padded] after the heads' RMS norm (weights float32 [dim] or None) and the rotation of their
+    first ``pairs`` pairs (i, i + pairs) by ``cos_sin`` [T, pairs, 2]; the gates' sigmoid (float32 [T, heads], or
+    None); and, if pools are given, keys (normed, rotated) and values written at ``slots``, the values mixed with
+    ``v_other`` (a view of the same type whose rows are ``v_other_stride`` apart) by the weight ``mix`` (float32 [1])
+    where it is given.  Heads are ``padded`` values wide in the queries and the pools, zeros at their end."""
+    _need(proj, "attention_prep proj", ndim=2)
+    t, w = proj.shape
+    if max(q_off + heads * dim, k_off + kv_heads * dim, v_off + kv_heads * vdim, g_off + (heads if gated else 0)) > w:
+        raise KernelError("attention_prep: the projection's rows are shorter than q, k, v and the gates")
+    for name, wt in (("q", q_weight), ("k", k_weight)):
+        if wt is not None:
+            _need(wt, f"attention_prep {name} norm weight", dtype=torch.float32, shape=(dim,))
+    if pairs:
+        _need(cos_sin, "attention_prep cos/sin", dtype=torch.float32, shape=(t, pairs, 2))
+    page_size = pool_slots = 0
+    if k_pool is not None:
+        _need(k_pool, "k_pool", dtype=proj.dtype, ndim=4)
+        units, kvh, page_size, hd = k_pool.shape
+        _need(v_pool, "v_pool", dtype=proj.dtype, shape=(units, kvh, hd, page_size))
+        if kvh != kv_heads or hd != padded:
+            raise KernelError(f"attention_prep: pools {tuple(k_pool.shape)} do not hold {kv_heads} heads of {padded}")
+        _need(slots, "attention_prep slots", dtype=torch.int32, shape=(t,))
+        pool_slots = units * page_size
+    if v_other is not None:
+        if v_other.dtype != proj.dtype or not v_other.is_cuda or v_other.stride(-1) != 1:
+            raise KernelError("attention_prep: the other layer's values must be of the projection's type")
+        _need(mix, "attention_prep mix", dtype=torch.float32)
+    q = torch.empty((t, heads * padded), dtype=proj.dtype, device=proj.device)
+    gate = torch.empty((t, heads), dtype=torch.float32, device=proj.device) if gated else None
+    check(load().fsie_attention_prep(proj.data_ptr(), w, q_off, k_off, v_off, g_off, heads, kv_heads, dim, vdim, padded,
+                                     _ptr(q_weight), _ptr(k_weight), float(eps), pairs, _ptr(cos_sin), _ptr(v_other),
+                                     int(v_other_stride), _ptr(mix), q.data_ptr(), _ptr(gate), _ptr(slots), _ptr(k_pool),
+                                     _ptr(v_pool), page_size, pool_slots, t, dtype_code(proj.dtype), _stream()))
+    return q, gate
+
+
+def gate_heads(x: torch.Tensor, padded: int, vdim: int, heads: int, gate: Optional[torch.Tensor]) -> torch.Tensor:
+    """[T, heads * vdim]: of every head of ``x`` [T, heads * padded] its first ``vdim`` values times ``gate``
+    (float32 [T, heads]; None: as they are)."""
+    _need(x, "gate_heads x", ndim=2)
+    t = x.shape[0]
+    if x.shape[1] != heads * padded or padded < vdim:
+        raise KernelError(f"gate_heads: rows of {x.shape[1]} are not {heads} heads of {padded}")
+    if gate is not None:
+        _need(gate, "gate_heads gate", dtype=torch.float32, shape=(t, heads))
+    y = torch.empty((t, heads * vdim), dtype=x.dtype, device=x.device)
+    check(load().fsie_gate_heads(x.data_ptr(), padded, _ptr(gate), y.data_ptr(), t, heads, vdim, dtype_code(x.dtype), _stream()))
+    return y

@@ -84,6 +84,14 @@ _SIGNATURES = {
                          _P], c_int),
     "fsie_head_gemm": ([_P, c_int64, c_int, c_int, _P, _P, c_int64, c_int, c_int, _P, c_int, c_int, c_int, c_int, c_int, _P],
                        c_int),
+    "fsie_rope_table_scaled": ([_P, _P, c_int, c_int, c_float, _P, _P], c_int),
+    "fsie_layer_norm": ([_P, _P, c_int, _P, c_int, _P, _P, _P, _P, _P, _P, _P, c_int, c_int, c_float, c_int, c_int, c_int, _P],
+                        c_int),
+    "fsie_pair_embedding": ([_P, _P, c_int, _P, _P, _P, c_int, _P, c_int, _P, c_int, c_int, c_int, c_int, c_int64, c_int64,
+                             c_float, _P], c_int),
+    "fsie_attention_prep": ([_P, c_int64, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, _P, _P, c_float,
+                             c_int, _P, _P, c_int64, _P, _P, _P, _P, _P, _P, c_int, c_int64, c_int, c_int, _P], c_int),
+    "fsie_gate_heads": ([_P, c_int, _P, _P, c_int, c_int, c_int, c_int, _P], c_int),
     "fsie_sample": ([_P, c_int, c_int, _P, _P, _P, _P, _P, _P], c_int),
 }
 

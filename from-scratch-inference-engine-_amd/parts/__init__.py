@@ -4,16 +4,16 @@ and the arrangement of a block."""
 from .base import (Block, FeedForward, HiddenState, Mixer, Norm, ParamDecl, Part, PositionEncoding,
                    known_parts, make_part, prepare_parts, register_part)
 from .attention import AttentionPlanner, GQAttention
-from .block import PreNormBlock, SandwichNormBlock
-from .embedding import LMHead, TokenEmbedding
+from .block import ParallelBlock, PreNormBlock, SandwichNormBlock
+from .embedding import LMHead, PairHashEmbedding, TokenEmbedding
 from .latent_attention import LatentAttention
 from .linear import Linear
 from .linear_attention import GatedLinearAttention
 from .mlp import SwiGLU
-from .norm import RMSNorm
+from .norm import LayerNorm, RMSNorm
 from .rope import NoPositionEncoding, RotaryEncoding
 
 __all__ = ["AttentionPlanner", "Block", "FeedForward", "GQAttention", "GatedLinearAttention", "HiddenState", "LMHead",
-           "LatentAttention", "Linear", "SandwichNormBlock", "Mixer", "NoPositionEncoding", "Norm", "ParamDecl", "Part", "PositionEncoding",
+           "LatentAttention", "LayerNorm", "Linear", "PairHashEmbedding", "ParallelBlock", "SandwichNormBlock", "Mixer", "NoPositionEncoding", "Norm", "ParamDecl", "Part", "PositionEncoding",
            "PreNormBlock", "RMSNorm", "RotaryEncoding", "SwiGLU", "TokenEmbedding", "known_parts",
            "make_part", "prepare_parts", "register_part"]

@@ -10,7 +10,7 @@ import torch
 
 from .. import ops
 from ..cache.manager import PagedNeed
-from ..ops.functions import ATTN_ITEM_INTS, ATTN_MERGE_INTS
+from ..ops.functions import ATTN_ITEM_INTS, ATTN_KEEP_WALK, ATTN_MERGE_INTS
 from ..ops.functions import GEMM_MFMA_SKINNY_BEST_M
 from .base import Mixer, Norm, ParamDecl, Part, PositionEncoding, register_part
 from .linear import Linear
@@ -43,10 +43,22 @@ class AttentionPlanner:
     # Compute units to fill with the workgroups of small items; None: those of the device.
     compute_units: Optional[int] = None
 
-    def __init__(self, n_heads: int, n_kv: int, head_dim: int, window: Optional[int]):
+    def __init__(self, n_heads: int, n_kv: int, head_dim: int, window: Optional[int], keep_first: int = 0):
+        """``keep_first`` (with a window): the first positions of a request stay visible to every later query.
+        Items say so in their last field (``ATTN_ITEM_KEEP``); an item whose window has left those keys behind
+        reads them first and then its own range (flag ``ATTN_KEEP_WALK``), and where a request's keys are split
+        over several items the kept keys are an item of their own that is merged with the rest."""
         self.n_heads, self.n_kv, self.head_dim, self.window = n_heads, n_kv, head_dim, window
-        self.key = ("attention", n_heads, n_kv, head_dim, window)
+        self.keep_first = int(keep_first) if window else 0
+        self.key = ("attention", n_heads, n_kv, head_dim, window, self.keep_first)
         self._geometry = {}
+
+    def _first_key(self, p: int):
+        """(first key of the window of the query at position p, kept keys that lie before it)."""
+        first = max(0, p - self.window + 1) if self.window else 0
+        if self.keep_first and first <= self.keep_first:
+            return 0, 0  # the kept keys and the window touch: one range, the mask does the rest
+        return first, (self.keep_first if first else 0)
 
     def geometry(self, mfma: bool):
         """(small_tokens, large_tokens, split_keys) of a kernel family."""
@@ -65,7 +77,9 @@ class AttentionPlanner:
 
     def uses_mfma(self, compute_dtype, page_size: int) -> bool:
         return (compute_dtype == torch.bfloat16 and self.head_dim % 16 == 0 and self.head_dim <= 256
-                and page_size % 4 == 0)
+                and page_size % 4 == 0 and (not self.keep_first or self.mfma_keeps_first))
+
+    mfma_keeps_first = False  # whether the matrix-core kernels read an item's kept first keys
 
     def _waves_for(self, keys: int, max_waves: int) -> int:
         """Waves of a workgroup for an item of ``keys`` keys: one per 128 keys, a power of two."""
@@ -81,7 +95,8 @@ class AttentionPlanner:
         for s in range(host.n_seqs):
             n, p = host.q_lens[s], host.past_lens[s]
             if n <= small_tokens:
-                keys.append(p + n - (max(0, p - self.window + 1) if self.window else 0))
+                first, kept = self._first_key(p)
+                keys.append(p + n - first + kept)
         return keys
 
     def split_keys(self, host, mfma: bool) -> int:
@@ -206,12 +221,15 @@ class AttentionPlanner:
         for s in range(host.n_seqs):
             if host.q_lens[s] > small_tokens:
                 return None
-            first_key = max(0, host.past_lens[s] - self.window + 1) if self.window else 0
+            first_key, kept = self._first_key(host.past_lens[s])
             keys = host.past_lens[s] + host.q_lens[s] - first_key
             mine = self._items_of(keys, split_keys, most)
             longest = max(longest, keys - (mine - 1) * split_keys)  # (the last item; the others have split_keys, if any)
             if mine > 1:
                 longest = max(longest, split_keys)
+                mine += 1 if kept else 0  # (the kept first keys are an item of their own)
+            elif kept:
+                longest = max(longest, keys + 32 * -(-kept // 32))
             n += mine
         if mfma:
             # items: a multiple of the number of requests and of a quarter of what gives every unit a
@@ -237,19 +255,24 @@ class AttentionPlanner:
         n_partial = 0
         for s in range(host.n_seqs):
             n, p, row0 = host.q_lens[s], host.past_lens[s], host.q_starts[s]
-            first_key = max(0, p - self.window + 1) if self.window else 0
+            first_key, kept = self._first_key(p)
+            keep = self.keep_first
             total = p + n
             n_splits = self._items_of(total - first_key, split_keys, most) if split_keys is not None else 1
             if n <= small_tokens and n_splits > 1:
                 base = n_partial
+                if kept:
+                    small.append((s, row0, n, p, 0, kept, base, keep))
+                    base += n
                 for i in range(n_splits):
                     kb = first_key + i * split_keys
-                    small.append((s, row0, n, p, kb, total if i == n_splits - 1 else kb + split_keys, base + i * n, 0))
+                    small.append((s, row0, n, p, kb, total if i == n_splits - 1 else kb + split_keys, base + i * n, keep))
+                n_splits += 1 if kept else 0
                 for t in range(n):
-                    merges.append((row0 + t, base + t, n_splits, n))
+                    merges.append((row0 + t, n_partial + t, n_splits, n))
                 n_partial += n_splits * n
             elif n <= small_tokens:
-                small.append((s, row0, n, p, first_key, total, -1, 0))
+                small.append((s, row0, n, p, first_key, total, -1, keep | ATTN_KEEP_WALK if keep else 0))
             else:
                 # (the short tile that a long portion may end with stays with the portion's other tiles:
                 # as a small item it would walk all the portion's keys in one workgroup a kv head, alone
@@ -262,14 +285,18 @@ class AttentionPlanner:
                 run[:, 2] = np.minimum(large_tokens, n - t0)
                 run[:, 3] = pos0
                 run[:, 4] = np.maximum(0, pos0 - self.window + 1) if self.window else 0
+                if self.keep_first:
+                    run[:, 4] = np.where(run[:, 4] <= self.keep_first, 0, run[:, 4])
                 run[:, 5] = pos0 + run[:, 2]
                 run[:, 6] = -1
-                run[:, 7] = 0
+                run[:, 7] = self.keep_first | ATTN_KEEP_WALK if self.keep_first else 0
                 large_runs.append(run)
         large = np.concatenate(large_runs) if large_runs else np.zeros((0, ATTN_ITEM_INTS), dtype=np.int64)
         waves = 1
         if mfma and small:
-            waves = self._waves_for(max(it[5] - it[4] for it in small), ops.attention_mfma_max_waves(self.head_dim))
+            waves = self._waves_for(max(it[5] - it[4] + (32 * -(-min(it[7] & ~ATTN_KEEP_WALK, it[4]) // 32)
+                                                            if it[7] & ATTN_KEEP_WALK else 0) for it in small),
+                                    ops.attention_mfma_max_waves(self.head_dim))
         if padded:
             # a captured graph launches fixed grids: pad with items and merges that do nothing
             n_items, waves, _ = host.pad[self.key]
@@ -358,7 +385,17 @@ class GQAttention(Mixer):
     1/sqrt(head_dim), output projection without bias (src/model/model.cpp:110-129,
     src/model/nn.cpp:151-226).  ``window`` = number of latest positions a query reads (None: all).
     ``sink=True``: a learned number per head (parameter ``sink``) whose exponential joins the softmax's
-    denominator; it has no key and no value.
+    denominator; it has no key and no value.  ``keep_first``: with a window, the first positions of a request
+    that every later query still reads.  ``scale``: the factor on the scores (None: 1/sqrt(head_dim)).
+    ``value_dim``: the size of a head's values where it is not the keys' (the cache and the attention kernels then
+    work on heads of ``padded`` values, the larger of the two rounded up to 16, zeros at their end).
+    ``gate=True``: the projection has one more row a head, and head h's result is multiplied by the sigmoid of
+    its row's product with x before the output projection.  ``value_mix``: "source" publishes this layer's
+    values of the step's tokens, "mixed" replaces its own by (1 - w) v + w v_source (parameter
+    ``value_mix_weight``, one number) before they are cached; both ends must agree in kv heads and value size.
+    With any of the last three, what stands between projection and attention is one kernel
+    (``ops.attention_prep``: head norms, rotation of the first ``rotary_dim`` values from the step's table, value
+    mixing, gates, cache write) and one after it (``ops.gate_heads``).
 
     What happens between the projection and attention, in this order: bias, ``q_norm`` / ``k_norm``
     (a norm as wide as a head, applied to every head through ``Norm.plain``; None: none), the
@@ -383,22 +420,39 @@ class GQAttention(Mixer):
 
     def __init__(self, hidden_size: int, n_heads: int, n_kv_heads: int, head_dim: int, qkv_bias: bool,
                  position: PositionEncoding, window: Optional[int] = None, q_norm: Optional[Norm] = None,
-                 k_norm: Optional[Norm] = None, sink: bool = False):
+                 k_norm: Optional[Norm] = None, sink: bool = False, keep_first: int = 0, scale: Optional[float] = None,
+                 value_dim: Optional[int] = None, gate: bool = False, value_mix: Optional[str] = None):
         if n_heads % n_kv_heads:
             raise ValueError(f"attention: heads {n_heads} must be a multiple of kv heads {n_kv_heads}")
-        if head_dim > 256:
-            raise ValueError(f"attention: head_dim {head_dim} is larger than the kernels take (256)")
+        self.value_dim = head_dim if value_dim is None else int(value_dim)
+        self.padded = head_dim if self.value_dim == head_dim else -(-max(head_dim, self.value_dim) // 16) * 16
+        if self.padded > 256 or self.value_dim < 1:
+            raise ValueError(f"attention: heads of {head_dim} (values {self.value_dim}) are larger than the kernels take (256)")
+        if value_mix not in (None, "source", "mixed"):
+            raise ValueError(f"attention: value_mix '{value_mix}' is neither 'source' nor 'mixed'")
+        if keep_first < 0 or (keep_first and not window):
+            raise ValueError("attention: keep_first goes with a window")
         self.hidden_size, self.n_heads, self.n_kv, self.head_dim = hidden_size, n_heads, n_kv_heads, head_dim
-        self.window = window
+        self.window, self.keep_first = window, int(keep_first)
         self.position = position
         self.q_norm, self.k_norm = q_norm, k_norm
-        self.q_dim, self.kv_dim = n_heads * head_dim, n_kv_heads * head_dim
-        self.qkv = Linear(hidden_size, self.q_dim + 2 * self.kv_dim, bias=qkv_bias)
-        self.o = Linear(self.q_dim, hidden_size)
-        self.scale = 1.0 / math.sqrt(head_dim)
+        self.has_gate, self.value_mix = bool(gate), value_mix
+        self.prepared = self.has_gate or value_mix is not None or self.value_dim != head_dim
+        if self.prepared:
+            if position.rotates and getattr(position, "layout", None) != "half":
+                raise ValueError("attention: with a gate, mixed values or values of another size the position encoding "
+                                 "must be the rotation of the pairs (i, i + rotary_dim / 2), or none")
+            if q_norm is not None and k_norm is not None and q_norm.eps != k_norm.eps:
+                raise ValueError("attention: the norms of the q and k heads must share their eps")
+        self.rot_pairs = (getattr(position, "rotary_dim", 0) // 2) if position.rotates else 0
+        self.q_dim, self.kv_dim, self.v_dim = n_heads * head_dim, n_kv_heads * head_dim, n_kv_heads * self.value_dim
+        self.qkv = Linear(hidden_size, self.q_dim + self.kv_dim + self.v_dim + (n_heads if gate else 0), bias=qkv_bias)
+        self.o = Linear(n_heads * self.value_dim, hidden_size)
+        self.scale = 1.0 / math.sqrt(head_dim) if scale is None else float(scale)
         self._planner: Optional[AttentionPlanner] = None
         self.has_sink = bool(sink)
         self.sink: Optional[torch.Tensor] = None
+        self.value_mix_weight: Optional[torch.Tensor] = None
 
     def sub_parts(self) -> Dict[str, Part]:
         parts: Dict[str, Part] = {"position": self.position}
@@ -410,12 +464,16 @@ class GQAttention(Mixer):
 
     # parameters -------------------------------------------------------------------------
     def param_decls(self) -> Dict[str, ParamDecl]:
-        decls = {"qkv_weight": ParamDecl((self.q_dim + 2 * self.kv_dim, self.hidden_size)),
-                 "o_weight": ParamDecl((self.hidden_size, self.q_dim))}
+        rows = self.qkv.out_features
+        decls = {"qkv_weight": ParamDecl((rows, self.hidden_size)),
+                 "o_weight": ParamDecl((self.hidden_size, self.n_heads * self.value_dim))}
         if self.qkv.has_bias:
-            decls["qkv_bias"] = ParamDecl((self.q_dim + 2 * self.kv_dim,), "vector", "bias")
+            decls["qkv_bias"] = ParamDecl((rows,), "vector", "bias")
         if self.has_sink:
             decls["sink"] = ParamDecl((self.n_heads,), "vector", "bias")
+        if self.value_mix is not None:
+            # (the source layer's number exists in checkpoints and is not used)
+            decls["value_mix_weight"] = ParamDecl((), "vector", "bias")
         return decls
 
     qkv_weight = property(lambda s: s.qkv.weight, lambda s, t: setattr(s.qkv, "weight", t))
@@ -432,11 +490,11 @@ class GQAttention(Mixer):
 
     # cache and plan ---------------------------------------------------------------------
     def cache_need(self) -> PagedNeed:
-        return PagedNeed(self.n_kv, self.head_dim, self.window)
+        return PagedNeed(self.n_kv, self.padded, self.window, self.keep_first if self.window else 0)
 
     def planner(self) -> AttentionPlanner:
         if self._planner is None:
-            self._planner = AttentionPlanner(self.n_heads, self.n_kv, self.head_dim, self.window)
+            self._planner = AttentionPlanner(self.n_heads, self.n_kv, self.padded, self.window, self.keep_first)
         return self._planner
 
     # compute ----------------------------------------------------------------------------
@@ -451,7 +509,7 @@ class GQAttention(Mixer):
     def _from_sums(self, x: torch.Tensor, ctx, cache, plan, table) -> Optional[torch.Tensor]:
         """Attention of a step of one token a request straight from the q/k/v product's partial sums
         (None: not such a step, or the kernels do not take the sizes)."""
-        if not (self.finish_qkv_in_attention and self.sink is None and table is not None and cache.writes and plan.mfma and plan.single
+        if not (self.finish_qkv_in_attention and self.sink is None and not self.keep_first and table is not None and cache.writes and plan.mfma and plan.single
                 and plan.n_small and not plan.n_large and not plan.n_long and x.dtype == torch.bfloat16
                 and ops.attention_mfma_qkv_ok(self.head_dim, cache.page_size)):
             return None
@@ -510,8 +568,41 @@ class GQAttention(Mixer):
             ops.rope_kv_write(qkv, ctx.positions, nh, nkv, hd, None, bias=bias, **store)  # (no rotation: bias, write)
         return qkv
 
+    def _forward_prepared(self, x: torch.Tensor, ctx, cache, plan) -> torch.Tensor:
+        """Gate, mixed values or values of another size than the keys: the fused projection, one kernel for all
+        that stands between it and attention, attention over heads of ``padded`` values, the gate."""
+        nh, nkv, hd, vd, pd = self.n_heads, self.n_kv, self.head_dim, self.value_dim, self.padded
+        proj = self.qkv(x)
+        k_off, v_off = self.q_dim, self.q_dim + self.kv_dim
+        g_off = v_off + self.v_dim
+        table = self.position.table(ctx) if self.rot_pairs else None
+        other, other_stride = None, 0
+        memo = ("attention values", nkv, vd)
+        if self.value_mix == "source":
+            ctx.memo[memo] = proj[:, v_off:v_off + self.v_dim]  # (a view: the projection lives as long as the step's memo)
+        elif self.value_mix == "mixed":
+            other = ctx.memo.get(memo)
+            if other is None:
+                raise RuntimeError("attention: no earlier layer of this step has published values to mix with")
+            other_stride = other.stride(0)
+        norm = self.q_norm if self.q_norm is not None else self.k_norm
+        store = dict(slots=cache.slots, k_pool=cache.k_pool, v_pool=cache.v_pool) if cache.writes else {}
+        q, gate = ops.attention_prep(proj, 0, k_off, v_off, g_off, nh, nkv, hd, vd, pd,
+                                     None if self.q_norm is None else self.q_norm.weight,
+                                     None if self.k_norm is None else self.k_norm.weight,
+                                     norm.eps if norm is not None else 0.0, self.rot_pairs, table, self.has_gate,
+                                     v_other=other, v_other_stride=other_stride,
+                                     mix=self.value_mix_weight if other is not None else None, **store)
+        out = paged_attention(q, nh * pd, cache, plan, nh, nkv, pd, self.window, self.scale, x.shape[0], sinks=self.sink,
+                              share_keys=self.share_keys)
+        if gate is not None or pd != vd:
+            out = ops.gate_heads(out, pd, vd, nh, gate)
+        return self.o.for_residual(out, ctx)
+
     def forward(self, x: torch.Tensor, ctx, cache) -> torch.Tensor:
         plan = ctx.plan(self.planner())
+        if self.prepared:
+            return self._forward_prepared(x, ctx, cache, plan)
         table = self._fused_table(ctx)
         out = self._from_sums(x, ctx, cache, plan, table)
         if out is not None:

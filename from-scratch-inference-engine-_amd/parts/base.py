@@ -48,14 +48,17 @@ class HiddenState:
     ``adds_partial_sums``, which the step's context then says in ``partial_sums_ok``) float32
     [S, T, H], partial sums of a matrix product to be added in order.  ``delta_norm``: a norm that the
     pending delta goes through before it is added (a layer that also norms its sublayers' outputs), or
-    None; the norm that folds the delta in applies it in the same pass."""
+    None; the norm that folds the delta in applies it in the same pass.  ``delta2``: a second pending delta of
+    the same kinds, left by a block whose mixer and feed-forward read the same stream (only norms that set
+    ``adds_two_deltas`` take it; the others refuse)."""
 
-    __slots__ = ("residual", "delta", "delta_norm")
+    __slots__ = ("residual", "delta", "delta_norm", "delta2")
 
     def __init__(self, residual: torch.Tensor, delta: Optional[torch.Tensor] = None, delta_norm=None):
         self.residual = residual
         self.delta = delta
         self.delta_norm = delta_norm
+        self.delta2 = None
 
 
 class Part:
@@ -108,6 +111,9 @@ class Norm(Part):
     kind = "norm"
     # True if the norm also takes a pending delta that comes as float32 partial sums [S, T, H]
     adds_partial_sums = False
+    # True if the norm adds a second pending delta (``HiddenState.delta2``) in the same pass, and offers
+    # ``pair(hidden, other, out_dtype)``: this norm's and another one's output of the same stream at once
+    adds_two_deltas = False
 
     def __call__(self, hidden: HiddenState, out_dtype: torch.dtype) -> torch.Tensor:
         raise NotImplementedError

@@ -56,3 +56,34 @@ class SandwichNormBlock(Block):
         if self.ffn is not None:
             x = self.ffn_norm(hidden, ctx.compute_dtype)
             hidden.delta, hidden.delta_norm = self.ffn.forward(x, ctx), self.ffn_post_norm
+
+
+@register_part("block", "parallel")
+class ParallelBlock(Block):
+    """Mixer and feed-forward side by side: x += mixer(norm1(x)) + ffn(norm2(x)), both norms of the same x.  The two
+    outputs stay pending in the hidden state as two deltas, and the norm that reads the stream next adds both in
+    the pass that normalises; this block's two norms are one pass as well (``Norm.pair``).  ``ffn=None``: the layer
+    has no feed-forward (and no second norm)."""
+
+    graph_safe = True
+
+    def __init__(self, mixer_norm: Norm, mixer: Mixer, ffn_norm: Optional[Norm] = None, ffn: Optional[FeedForward] = None):
+        if (ffn is None) != (ffn_norm is None):
+            raise ValueError("parallel block: a feed-forward comes with its norm, or neither")
+        if not mixer_norm.adds_two_deltas or (ffn_norm is not None and not ffn_norm.adds_two_deltas):
+            raise ValueError("parallel block: its norms must add two pending deltas and come as a pair (layer_norm does)")
+        self.mixer_norm, self.mixer, self.ffn_norm, self.ffn = mixer_norm, mixer, ffn_norm, ffn
+
+    def sub_parts(self) -> Dict[str, Part]:
+        parts = {"mixer_norm": self.mixer_norm, "mixer": self.mixer}
+        if self.ffn is not None:
+            parts.update(ffn_norm=self.ffn_norm, ffn=self.ffn)
+        return parts
+
+    def forward(self, hidden: HiddenState, ctx, cache) -> None:
+        if self.ffn is None:
+            hidden.delta = self.mixer.forward(self.mixer_norm(hidden, ctx.compute_dtype), ctx, cache)
+            return
+        a, b = self.mixer_norm.pair(hidden, self.ffn_norm, ctx.compute_dtype)
+        hidden.delta = self.mixer.forward(a, ctx, cache)
+        hidden.delta2 = self.ffn.forward(b, ctx)

@@ -28,6 +28,48 @@ class TokenEmbedding(Part):
     def forward(self, ids: torch.Tensor) -> torch.Tensor:
         return ops.embedding(self.weight, ids)
 
+    def cache_need(self):
+        """What the embedding keeps for a request between steps (a need of ``cache.needs``), or None."""
+        return None
+
+    def embed(self, ctx, cache) -> torch.Tensor:
+        """The float32 stream of the step's tokens; ``cache`` is the view of what ``cache_need`` asked for."""
+        return self.forward(ctx.token_ids)
+
+
+class PairHashEmbedding(TokenEmbedding):
+    """x[t] = table[id_t] * scale + pairs[(id_{t-1} * mul_prev + id_t * mul_cur) mod buckets]: a second table of
+    ``buckets`` + 1 rows, addressed by a hash of the token and the one before it; a request's first token takes the
+    last row.  The token before a portion's first one comes from the request's state slot (one int32: the latest
+    id + 1, zero when the request starts), which the step brings up to date, so portions, single tokens and
+    sampled ids that only the device knows all see the right neighbour."""
+
+    graph_safe = True
+
+    def __init__(self, vocab_size: int, hidden_size: int, buckets: int, mul_prev: int, mul_cur: int, scale: float = 1.0):
+        super().__init__(vocab_size, hidden_size)
+        if buckets < 1:
+            raise ValueError(f"pair embedding: buckets {buckets} must be positive")
+        self.buckets, self.mul_prev, self.mul_cur, self.scale = int(buckets), int(mul_prev), int(mul_cur), float(scale)
+        self.pair_weight = None
+
+    def param_decls(self) -> Dict[str, ParamDecl]:
+        return {"weight": ParamDecl((self.vocab_size, self.hidden_size)),
+                "pair_weight": ParamDecl((self.buckets + 1, self.hidden_size))}
+
+    def cache_need(self):
+        from ..cache.needs import StateNeed
+
+        return StateNeed((1,), "int32")
+
+    def forward(self, ids: torch.Tensor) -> torch.Tensor:
+        raise RuntimeError("pair embedding: the step's tables and the requests' state are needed (embed)")
+
+    def embed(self, ctx, cache) -> torch.Tensor:
+        if cache is None or cache.state is None:
+            raise RuntimeError("pair embedding: no state slots (the model did not ask for the embedding's cache need)")
+        return ops.pair_embedding(self.weight, self.pair_weight, ctx.token_ids, ctx.q_starts, ctx.seq_slots, cache.state,
+                                  self.mul_prev, self.mul_cur, self.scale)
 
 class LMHead(Part):
     """logits = x . W^T in float32, no bias (src/model/model.cpp:144-148).  With tied embeddings

@@ -21,8 +21,8 @@ class LatentAttention(Mixer):
     ``rot_dim`` that the position encoding turns.  Keys and values through a latent: c = rmsnorm(first
     ``kv_rank`` rows of W_dkv x); the last ``rot_dim`` rows, turned, are a key part that all heads share.
     Head h's key is [W_uk,h c | shared part], its value W_uv,h c, the score their product with the query
-    times ``scale``, the softmax causal with a sink per head (``sink=True``), the head's result multiplied by
-    sigmoid(W_g x)_h (``gate=True``), and W_o over the heads.
+    times ``scale``, the softmax causal (over the latest ``window`` positions only, if given) with a sink per head
+    (``sink=True``), the head's result multiplied by sigmoid(W_g x)_h (``gate=True``), and W_o over the heads.
 
     Only c and the shared part are cached: one row of ``width`` values a token (their sum rounded up to 16,
     zeros at the end; up to 256 values the matrix-core kernels serve bfloat16, wider rows up to 512 go to the
@@ -40,14 +40,21 @@ class LatentAttention(Mixer):
 
     def __init__(self, hidden_size: int, n_heads: int, head_dim: int, rot_dim: int, value_dim: int, kv_rank: int,
                  q_rank: int, scale: float, norm_eps: float, position: PositionEncoding, own_latent: bool = True,
-                 sink: bool = True, gate: bool = True):
+                 sink: bool = True, gate: bool = True, window: Optional[int] = None):
         self.width = -(-(kv_rank + rot_dim) // 16) * 16
         if self.width > MAX_WIDTH:
             raise ValueError(f"latent attention: kv_rank {kv_rank} + rot_dim {rot_dim} is more than the attention "
                              f"kernels take in a cache row ({MAX_WIDTH})")
         self.rot_pairs = (getattr(position, "rotary_dim", 0) // 2) if position.rotates else 0
-        if position.rotates and (getattr(position, "layout", None) != "interleaved" or 2 * self.rot_pairs > rot_dim):
-            raise ValueError("latent attention: the position encoding must turn neighbouring pairs within rot_dim")
+        layout = getattr(position, "layout", None)
+        if position.rotates and (layout not in ("interleaved", "half") or 2 * self.rot_pairs > rot_dim):
+            raise ValueError("latent attention: the position encoding must turn pairs (neighbours, or value i with "
+                             "value i + rotary_dim / 2) within rot_dim")
+        # what the kernels are told: a positive number of neighbouring pairs, a negative one of pairs (i, i + pairs)
+        self.kernel_pairs = -self.rot_pairs if layout == "half" else self.rot_pairs
+        if window is not None and window < 1:
+            raise ValueError("latent attention: window must be >= 1")
+        self.window = window
         self.hidden_size, self.n_heads, self.head_dim, self.rot_dim = hidden_size, n_heads, head_dim, rot_dim
         self.value_dim, self.kv_rank, self.q_rank = value_dim, kv_rank, q_rank
         self.scale, self.norm_eps, self.position = float(scale), float(norm_eps), position
@@ -96,11 +103,11 @@ class LatentAttention(Mixer):
         return self.down.drop_copy() + self.o.drop_copy()
 
     def cache_need(self) -> Optional[PagedNeed]:
-        return PagedNeed(1, self.width, None) if self.own_latent else None
+        return PagedNeed(1, self.width, self.window) if self.own_latent else None
 
     def planner(self) -> AttentionPlanner:
         if self._planner is None:
-            self._planner = AttentionPlanner(self.n_heads, 1, self.width, None)
+            self._planner = AttentionPlanner(self.n_heads, 1, self.width, self.window)
         return self._planner
 
     def forward(self, x: torch.Tensor, ctx, cache) -> torch.Tensor:
@@ -112,16 +119,16 @@ class LatentAttention(Mixer):
         table = self.position.table(ctx) if self.rot_pairs else None
         p = self.down(x)
         pools = dict(slots=cache.slots, k_pool=cache.k_pool, v_pool=cache.v_pool) if self.own_latent else {}
-        cq, gate = ops.latent_prep(p, 0, self.q_rank, self.q_rank, self.kv_rank, self.rot_dim, self.rot_pairs,
+        cq, gate = ops.latent_prep(p, 0, self.q_rank, self.q_rank, self.kv_rank, self.rot_dim, self.kernel_pairs,
                                    self.q_rank + self.kv_rows, self.gate_rows, self.q_norm_weight, self.kv_norm_weight,
                                    self.norm_eps, table, **pools)
         q = self.uq(cq)
         # the queries as attention over the cached rows takes them: [W_uk,h^T q_h | turned part | zeros]
         qa = torch.empty((t, h * width), dtype=x.dtype, device=x.device)
         ops.head_gemm(q, 0, self.q_head, self._uk_by_head, qa, 0, width)
-        ops.rope_pairs(q, self.head_dim, self.q_head, qa, self.kv_rank, width, h, self.rot_dim, self.rot_pairs,
+        ops.rope_pairs(q, self.head_dim, self.q_head, qa, self.kv_rank, width, h, self.rot_dim, self.kernel_pairs,
                        width - self.kv_rank, table)
-        mixed = paged_attention(qa, h * width, cache, plan, h, 1, width, None, self.scale, t, sinks=self.sink)
+        mixed = paged_attention(qa, h * width, cache, plan, h, 1, width, self.window, self.scale, t, sinks=self.sink)
         y = torch.empty((t, h * self.value_dim), dtype=x.dtype, device=x.device)
         ops.head_gemm(mixed, 0, width, self._uv_by_head, y, 0, self.value_dim, gate=gate if self.has_gate else None)
         return self.o.for_residual(y, ctx)

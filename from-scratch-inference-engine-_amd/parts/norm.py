@@ -1,4 +1,4 @@
-"""RMSNorm, fused with the residual sum."""
+"""RMSNorm and layer norm, fused with the residual sum."""
 
 from __future__ import annotations
 
@@ -8,6 +8,12 @@ import torch
 
 from .. import ops
 from .base import HiddenState, Norm, ParamDecl, register_part
+
+
+def _no_second_delta(hidden: HiddenState, name: str) -> None:
+    if hidden.delta2 is not None:
+        raise RuntimeError(f"{name}: the stream has a second pending delta (a block whose sublayers read the same "
+                           f"stream came before), which this norm does not add")
 
 
 @register_part("norm", "rms_norm")
@@ -40,6 +46,7 @@ class RMSNorm(Norm):
             self._offset_added = True
 
     def __call__(self, hidden: HiddenState, out_dtype: torch.dtype) -> torch.Tensor:
+        _no_second_delta(hidden, "rms_norm")
         delta, post = hidden.delta, hidden.delta_norm
         hidden.delta = hidden.delta_norm = None
         if delta is not None and post is not None:
@@ -49,6 +56,7 @@ class RMSNorm(Norm):
                            write_back=delta is not None)
 
     def rows(self, hidden: HiddenState, rows: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
+        _no_second_delta(hidden, "rms_norm")
         if hidden.delta is not None and hidden.delta_norm is not None:
             post = hidden.delta_norm
             return ops.sandwich_norm(hidden.residual, hidden.delta, post.weight, post.eps, self.weight, self.eps,
@@ -57,3 +65,50 @@ class RMSNorm(Norm):
 
     def plain(self, x: torch.Tensor, out=None) -> torch.Tensor:
         return ops.rmsnorm_plain(x, self.weight, self.eps, out=out)
+
+
+@register_part("norm", "layer_norm")
+class LayerNorm(Norm):
+    """y = (x - mean(x)) / sqrt(var(x) + eps) * w + b with x = residual + pending deltas, the variance the mean of
+    the squared deviations, everything in float32.  It adds up to two pending deltas (each whole or as float32
+    partial sums), and ``pair`` gives this norm's and another layer norm's output of the same stream from one
+    pass: they share mean and variance and differ in weight and bias only."""
+
+    adds_partial_sums = True
+    adds_two_deltas = True
+    graph_safe = True
+
+    def __init__(self, hidden_size: int, eps: float):
+        self.hidden_size = hidden_size
+        self.eps = float(eps)
+        self.weight = None
+        self.bias = None
+
+    def param_decls(self) -> Dict[str, ParamDecl]:
+        return {"weight": ParamDecl((self.hidden_size,), "vector", "norm"),
+                "bias": ParamDecl((self.hidden_size,), "vector", "bias")}
+
+    @staticmethod
+    def _take(hidden: HiddenState, clear: bool):
+        if hidden.delta_norm is not None:
+            raise RuntimeError("layer_norm: a pending delta with a norm of its own is not taken")
+        deltas = hidden.delta, hidden.delta2
+        if clear:
+            hidden.delta = hidden.delta2 = None
+        return deltas
+
+    def __call__(self, hidden: HiddenState, out_dtype: torch.dtype) -> torch.Tensor:
+        d1, d2 = self._take(hidden, True)
+        return ops.layer_norm(hidden.residual, self.weight, self.bias, self.eps, out_dtype, delta=d1, delta2=d2,
+                              write_back=d1 is not None or d2 is not None)
+
+    def pair(self, hidden: HiddenState, other: "LayerNorm", out_dtype: torch.dtype):
+        if not isinstance(other, LayerNorm) or other.eps != self.eps or other.hidden_size != self.hidden_size:
+            raise ValueError("layer_norm: a pair is two layer norms of one width and eps")
+        d1, d2 = self._take(hidden, True)
+        return ops.layer_norm(hidden.residual, self.weight, self.bias, self.eps, out_dtype, delta=d1, delta2=d2,
+                              weight2=other.weight, bias2=other.bias, write_back=d1 is not None or d2 is not None)
+
+    def rows(self, hidden: HiddenState, rows: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
+        d1, d2 = self._take(hidden, False)
+        return ops.layer_norm(hidden.residual, self.weight, self.bias, self.eps, out_dtype, delta=d1, delta2=d2, rows=rows)

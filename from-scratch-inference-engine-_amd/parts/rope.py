@@ -2,6 +2,7 @@
 
 from __future__ import annotations
 
+import math
 from typing import Optional
 
 import numpy as np
@@ -18,11 +19,19 @@ class RotaryEncoding(PositionEncoding):
     (src/model/nn.cpp:110-149).  Where the whole head rotates it also offers the step's table of
     cosines and sines, from which a mixer's own kernels rotate.  ``layout="interleaved"``: the pairs are
     neighbours (2i, 2i + 1) instead, the frequencies the same; ``table`` gives a mixer the step's cosines
-    and sines for its own kernels, ``rotate`` turns the first ``rotary_dim`` values of every q and k head."""
+    and sines for its own kernels, ``rotate`` turns the first ``rotary_dim`` values of every q and k head.
+
+    ``stretch`` = (factor, original, fast, slow) rescales the frequencies for contexts beyond ``original``
+    positions: with dim(t) = rotary_dim * ln(original / (2 pi t)) / (2 ln theta), lo = max(floor(dim(fast)), 0),
+    hi = min(ceil(dim(slow)), rotary_dim - 1) and ramp_i = clamp((i - lo) / max(hi - lo, 0.001), 0, 1), pair i
+    turns at f_i / factor * ramp_i + f_i * (1 - ramp_i) (fast pairs stay, slow pairs are divided by the factor,
+    a ramp between), and every cosine and sine is multiplied by 0.1 * ln(factor) + 1.  That factor only exists
+    in the table: ``rotate`` refuses where it would have to compute the angles itself."""
 
     graph_safe = True
 
-    def __init__(self, head_dim: int, theta: float, rotary_dim: Optional[int] = None, layout: str = "half"):
+    def __init__(self, head_dim: int, theta: float, rotary_dim: Optional[int] = None, layout: str = "half",
+                 stretch: Optional[tuple] = None):
         if layout not in ("half", "interleaved"):
             raise ValueError(f"rope: unknown layout '{layout}' (half or interleaved)")
         self.layout = layout
@@ -32,19 +41,42 @@ class RotaryEncoding(PositionEncoding):
         if self.rotary_dim % 2 or not 0 < self.rotary_dim <= head_dim:
             raise ValueError(f"rope: rotary_dim {self.rotary_dim} must be even and within head_dim {head_dim}")
         self.inv_freq = None
+        self.magnitude = 1.0
+        self.stretch = None
+        if stretch is not None:
+            factor, original, fast, slow = (float(v) for v in stretch)
+            if not (factor >= 1.0 and original > 0 and fast > 0 and slow > 0 and self.theta > 1.0):
+                raise ValueError(f"rope: stretch {stretch} needs factor >= 1 and positive original, fast and slow")
+            self.stretch = (factor, original, fast, slow)
+            self.magnitude = 0.1 * math.log(factor) + 1.0
+
+    def frequencies(self) -> np.ndarray:
+        """float64 [rotary_dim / 2]: the angle a position adds to each pair."""
+        dims = self.rotary_dim
+        i = np.arange(dims // 2, dtype=np.float64)
+        freq = np.power(np.float64(self.theta), -2.0 * i / dims)
+        if self.stretch is None:
+            return freq
+        factor, original, fast, slow = self.stretch
+
+        def dim_of(turns: float) -> float:
+            return dims * math.log(original / (2.0 * math.pi * turns)) / (2.0 * math.log(self.theta))
+
+        lo = max(math.floor(dim_of(fast)), 0)
+        hi = min(math.ceil(dim_of(slow)), dims - 1)
+        ramp = np.clip((i - lo) / max(hi - lo, 0.001), 0.0, 1.0)
+        return freq / factor * ramp + freq * (1.0 - ramp)
 
     def prepare(self, device, compute_dtype) -> None:
-        i = np.arange(self.rotary_dim // 2, dtype=np.float64)
-        table = np.power(np.float64(self.theta), -2.0 * i / self.rotary_dim)
-        self.inv_freq = torch.from_numpy(table).to(device)
+        self.inv_freq = torch.from_numpy(self.frequencies()).to(device)
 
     def table(self, ctx) -> torch.Tensor:
         """The cosines and sines of this step's positions: the same in every layer, made by the
         first one that asks."""
-        key = ("rope cos/sin", self.theta, self.rotary_dim)
+        key = ("rope cos/sin", self.theta, self.rotary_dim, self.stretch)
         table = ctx.memo.get(key)
         if table is None:
-            table = ctx.memo[key] = ops.rope_table(ctx.positions, self.inv_freq)
+            table = ctx.memo[key] = ops.rope_table(ctx.positions, self.inv_freq, self.magnitude)
         return table
 
     def rotation_table(self, head_dim, ctx):
@@ -57,6 +89,8 @@ class RotaryEncoding(PositionEncoding):
                            head_dim, self.table(ctx))
             return
         cos_sin = self.table(ctx) if self.rotary_dim == head_dim and head_dim % 8 == 0 else None
+        if cos_sin is None and self.magnitude != 1.0:
+            raise NotImplementedError("rope: a stretched rotation of part of a head exists as a table only")
         ops.rope_kv_write(qkv, ctx.positions, n_heads, n_kv, head_dim, self.inv_freq, cos_sin=cos_sin)
 
 
