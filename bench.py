@@ -252,12 +252,30 @@ def gilozen_shape(width: int, ff: int, layers: int, vocab: int) -> dict:
             "layers": out}
 
 
+def botulorn_shape(width: int, ff: int, layers: int, vocab: int) -> dict:
+    """A Botulorn configuration of real layer sizes: attention through a latent and grouped-query attention in
+    turn (windows of 1,024 positions, the latter keeping a request's first four), every layer with a gated
+    feed-forward beside its mixer."""
+    heads = width // 128
+    stretch = {"factor": 8.0, "original": 1024, "fast": 32.0, "slow": 1.0}
+    latent = {"heads": heads, "dim": 64, "rot_dim": 64, "vdim": 128, "kv_rank": 192, "q_rank": width // 2 + 256,
+              "scale": 128 ** -0.5, "mask": {"size": 1024}, "rot": {"base": 500000.0, "dims": 64, "scaling": stretch}}
+    gqa = {"heads": heads, "kv_heads": max(1, width // 512), "dim": 128, "vdim": 128, "scale": 128 ** -0.5, "v_mix": True,
+           "mask": {"size": 1024, "keep_first": 4}, "rot": {"base": 500000.0, "dims": 64, "scaling": stretch}}
+    out = [{"type": "latent_attention" if i % 2 == 0 else "attention", "mixer": dict(latent if i % 2 == 0 else gqa),
+            "mlp": {"kind": "dense", "ff": ff}} for i in range(layers)]
+    return {"architecture": "Botulorn", "width": width, "vocab": vocab, "norm": {"eps": 1e-5},
+            "embedding": {"scale": width ** 0.5, "bigram": {"buckets": 65521, "mul_prev": 1000003, "mul_cur": 7}},
+            "layers": out}
+
+
+DESIGN_SHAPES = {"gilozen": gilozen_shape, "botulorn": botulorn_shape}
 DESIGN_SIZES = {"2048": (2048, 8192, 9, 32000), "4096": (4096, 14336, 9, 32000)}  # width, ff, layers, vocab
 
 
 def design_comparison(args) -> int:
-    """--workload gilozen: prefill (one prompt of 2,048 tokens in one step) and decode (batches of 8 and 64 at a
-    context of 512, from captured graphs) of Gilozen at two real layer sizes with random weights, beside a Qwen2
+    """--workload gilozen | botulorn: prefill (one prompt of 2,048 tokens in one step) and decode (batches of 8 and 64 at a
+    context of 512, from captured graphs) of the named design at two real layer sizes with random weights, beside a Qwen2
     model of the same width, feed-forward, layers and vocabulary (grouped-query attention, 128 values a head, four
     query heads a key/value head) through the same step function.  One JSON line."""
     import torch
@@ -276,7 +294,7 @@ def design_comparison(args) -> int:
                 "num_hidden_layers": layers, "num_attention_heads": width // 128, "num_key_value_heads": width // 512,
                 "head_dim": 128, "intermediate_size": ff, "vocab_size": vocab, "rope_theta": 500000.0,
                 "rms_norm_eps": 1e-5, "tie_word_embeddings": False, "max_position_embeddings": 8192}
-        for name, raw in (("gilozen", gilozen_shape(width, ff, layers, vocab)), ("qwen2", qwen)):
+        for name, raw in ((args.workload, DESIGN_SHAPES[args.workload](width, ff, layers, vocab)), ("qwen2", qwen)):
             model = Model.from_random(parse_config(raw), seed=0, dtype=dtype)
             pages_each = (512 + args.warmup + args.steps) // 16 + 2  # a decoding request's context and every step after it
             runner = Runner(model, page_size=16, num_pages=64 * max(40, pages_each) + 160, max_requests=64)
@@ -316,7 +334,7 @@ def design_comparison(args) -> int:
             print(f"[bench] width {width} {name}: " + ", ".join(f"{k} {v:.3f}" for k, v in row.items()), file=sys.stderr, flush=True)
             del runner, model
             torch.cuda.empty_cache()
-    print(json.dumps({"metric": "Gilozen beside Qwen2 at equal sizes: prefill tok/s @ 2,048 tokens, decode tok/s @ batch 8 and 64, context 512",
+    print(json.dumps({"metric": f"{args.workload.capitalize()} beside Qwen2 at equal sizes: prefill tok/s @ 2,048 tokens, decode tok/s @ batch 8 and 64, context 512",
                       "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "dtype": args.dtype,
                       "data": "synthetic: random weights N(0,0.02), uniform random token ids",
                       "sizes": {k: dict(zip(("width", "ff", "layers", "vocab"), DESIGN_SIZES[k])) for k in results},
@@ -341,13 +359,13 @@ def main() -> int:
     ap.add_argument("--no-tune", action="store_true", help="leave the library's kernel choice for prefill to its heuristic")
     ap.add_argument("--no-streamed-copies", action="store_true",
                     help="do not keep the large weights a second time in the order of the matrix instruction's fragments")
-    ap.add_argument("--design-sizes", default="2048,4096", help="--workload gilozen: widths to run (2048, 4096)")
-    ap.add_argument("--design-phases", default="prefill,decode", help="--workload gilozen: what to time (for a trace of one phase)")
-    ap.add_argument("--workload", choices=["decode", "mixed", "long-prefill", "gilozen"], default="decode",
+    ap.add_argument("--design-sizes", default="2048,4096", help="--workload gilozen | botulorn: widths to run (2048, 4096)")
+    ap.add_argument("--design-phases", default="prefill,decode", help="--workload gilozen | botulorn: what to time (for a trace of one phase)")
+    ap.add_argument("--workload", choices=["decode", "mixed", "long-prefill", "gilozen", "botulorn"], default="decode",
                     help="decode: the default run.  mixed: --requests prompts of --min-prompt to --max-prompt tokens, "
                          "--outputs tokens each, through the scheduler (made for --shape 14b).  "
                          "long-prefill: one prompt of --prefill-tokens tokens in portions of the token budget "
-                         "(made for --shape 32b).  gilozen: the Gilozen design beside Qwen2 at equal layer sizes")
+                         "(made for --shape 32b).  gilozen, botulorn: that design beside Qwen2 at equal layer sizes")
     ap.add_argument("--requests", type=int, default=32)
     ap.add_argument("--min-prompt", type=int, default=128)
     ap.add_argument("--max-prompt", type=int, default=4096)
@@ -373,7 +391,7 @@ def main() -> int:
         enable_library_tuning()  # the first prefill times the library's kernels for its shapes
         fill_rows = padded_tokens  # and steps that are not decode steps are filled up to the timed row counts
 
-    if args.workload == "gilozen":
+    if args.workload in DESIGN_SHAPES:
         return design_comparison(args)
     shape_name, shape = SHAPES[args.shape]
     raw = dict(shape)

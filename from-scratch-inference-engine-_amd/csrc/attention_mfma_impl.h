@@ -144,6 +144,11 @@ __global__ __launch_bounds__(QKV && MAXW == 1 ? 256 : 64 * MAXW) __attribute__((
     int key_end = item[FSIE_ATTN_ITEM_KEND];
     const int partial_base = item[FSIE_ATTN_ITEM_PARTIAL];
     if (n_q <= 0) return;  // padding item
+    // The first keys of the request that a window keeps: seen whatever the window says.  An item told to
+    // (FSIE_ATTN_KEEP_WALK) reads those that lie before its own range too, [0, prefix_end), as blocks of
+    // their own ahead of the range's blocks.
+    const int keep = item[FSIE_ATTN_ITEM_KEEP] & ~FSIE_ATTN_KEEP_WALK;
+    const int prefix_end = (item[FSIE_ATTN_ITEM_KEEP] & FSIE_ATTN_KEEP_WALK) ? min(keep, key_begin) : 0;
     // QKV: the item whose keys end with the request's new one walks the cache up to it and takes
     // the new key and value from the sums
     const bool owner = QKV && pos0 >= key_begin && pos0 < key_end;
@@ -293,7 +298,11 @@ __global__ __launch_bounds__(QKV && MAXW == 1 ? 256 : 64 * MAXW) __attribute__((
     const uint32_t page_magic = 0xFFFFFFFFu / static_cast<uint32_t>(page_size) + 1u;
     // this wave's run of key blocks
     const int kb_first = key_begin & ~31;
-    const int n_blocks = (key_end - kb_first + 31) >> 5;
+    // The walk runs over block coordinates: from kb_first on a coordinate is the key itself; the blocks of
+    // the kept first keys stand before that, from walk_first on, and coordinate u there is key u - walk_first.
+    const int pre_len = (prefix_end + 31) & ~31;
+    const int walk_first = kb_first - pre_len;
+    const int n_blocks = ((key_end - kb_first + 31) >> 5) + (pre_len >> 5);
     // an item uses one wave per 4 blocks (128 keys) of its own when it has one query tile, per 16
     // blocks (512 keys) when it has several, however many waves the launch has: how its keys are
     // split depends on the item alone
@@ -304,7 +313,7 @@ __global__ __launch_bounds__(QKV && MAXW == 1 ? 256 : 64 * MAXW) __attribute__((
     // idle if there is one (else for the first); n_runs = waves whose results are combined
     const int new_key_wave = owner && n_active < n_waves ? n_active : 0;
     const int n_runs = owner && n_active < n_waves ? n_active + 1 : n_active;
-    const int kb_begin = kb_first + wave * per_wave * 32;
+    const int kb_begin = walk_first + wave * per_wave * 32;
     const int kb_end = min(key_end, kb_begin + per_wave * 32);
     // the keys (A operand of the scores) and values (A operand of the second product) of a block
     struct Block {
@@ -323,8 +332,11 @@ __global__ __launch_bounds__(QKV && MAXW == 1 ? 256 : 64 * MAXW) __attribute__((
     };
     struct Asked {
         int page[4], idx[4], key[4];
+        int limit;  // keys from here on do not belong to the block's range
     };
     auto ask_pages = [&](int kb, Asked& p) {
+        p.limit = kb >= kb_first ? key_end : prefix_end;
+        kb = kb >= kb_first ? kb : kb - walk_first;
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
             p.key[t] = kb + 8 * (c >> 2) + 4 * t + (c & 3);
@@ -339,7 +351,7 @@ __global__ __launch_bounds__(QKV && MAXW == 1 ? 256 : 64 * MAXW) __attribute__((
     auto place = [&](const Asked& p, Where& at) {
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            const bool ok = p.key[i] < key_end && p.idx[i] < max_pages && p.page[i] >= 0;
+            const bool ok = p.key[i] < p.limit && p.idx[i] < max_pages && p.page[i] >= 0;
             const int64_t head = (static_cast<int64_t>(ok ? p.page[i] : 0) * n_kv + kvh) * head_stride;
             const int off = ok ? p.key[i] - p.idx[i] * page_size : 0;
             if (i < 2) at.k[i] = head + static_cast<int64_t>(off) * HD + (X32 ? 8 : 4) * G;
@@ -379,7 +391,9 @@ __global__ __launch_bounds__(QKV && MAXW == 1 ? 256 : 64 * MAXW) __attribute__((
         }
     };
     auto compute_block = [&](int kb, const Block& blk) {
-        const bool full = kb >= key_begin && kb + 32 <= key_end && kb + 31 <= pos0 &&
+        const bool kept_block = kb < kb_first;  // a block of the kept first keys (the same for the whole wave)
+        if (kept_block) kb -= walk_first;
+        const bool full = !kept_block && kb >= key_begin && kb + 32 <= key_end && kb + 31 <= pos0 &&
                           (window <= 0 || kb > pos0 + n_q - 1 - window);  // the same for the whole wave
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt) {
@@ -412,8 +426,9 @@ __global__ __launch_bounds__(QKV && MAXW == 1 ? 256 : 64 * MAXW) __attribute__((
 #pragma unroll
                     for (int r = 0; r < 4; ++r) {
                         const int key = kb + 8 * G + 4 * t + r;
-                        const bool vis = rvalid[nt] && key >= key_begin && key < key_end && key <= rpos[nt] &&
-                                         (window <= 0 || key > rpos[nt] - window);
+                        const bool in_range = kept_block ? key < prefix_end : (key >= key_begin && key < key_end);
+                        const bool vis = rvalid[nt] && in_range && key <= rpos[nt] &&
+                                         (window <= 0 || key > rpos[nt] - window || key < keep);
                         sv[t * 4 + r] = vis ? st[t][r] * scale2 : -INFINITY;
                         m_loc = fmaxf(m_loc, sv[t * 4 + r]);
                     }

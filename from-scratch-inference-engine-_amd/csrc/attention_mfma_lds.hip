@@ -123,6 +123,20 @@ __global__ __launch_bounds__(kLdsThreads) __attribute__((amdgpu_waves_per_eu(HDT
     // the workgroup's keys: from the first tile's first to the last tile's last
     const int wg_begin = items[static_cast<int64_t>(first) * FSIE_ATTN_ITEM_INTS + FSIE_ATTN_ITEM_KBEGIN] & ~(kLdsKeys - 1);
     const int wg_end = items[static_cast<int64_t>(first + n_tiles - 1) * FSIE_ATTN_ITEM_INTS + FSIE_ATTN_ITEM_KEND];
+    // The first keys of the request that a window keeps are seen whatever the window says.  Where the group's
+    // first tile starts beyond them, the workgroup reads them as blocks of their own before its range (the
+    // loop's coordinate u < wg_begin is key u - walk_first); where the range starts at key 0 they are part of it,
+    // and a later tile of the group whose own range starts beyond them sees them there (kept_in_range).
+    const int keep_raw = __builtin_amdgcn_readfirstlane(item[FSIE_ATTN_ITEM_KEEP]);
+    const int keep = keep_raw & ~FSIE_ATTN_KEEP_WALK;
+    const int kept_before = (keep_raw & FSIE_ATTN_KEEP_WALK) ? min(keep, key_begin) : 0;  // this wave's, before its range
+    const int first_raw = items[static_cast<int64_t>(first) * FSIE_ATTN_ITEM_INTS + FSIE_ATTN_ITEM_KEEP];
+    const int wg_kept = (first_raw & FSIE_ATTN_KEEP_WALK)
+                            ? min(first_raw & ~FSIE_ATTN_KEEP_WALK,
+                                  items[static_cast<int64_t>(first) * FSIE_ATTN_ITEM_INTS + FSIE_ATTN_ITEM_KBEGIN])
+                            : 0;
+    const int walk_first = wg_begin - ((wg_kept + kLdsKeys - 1) & ~(kLdsKeys - 1));
+    const int kept_in_range = wg_kept > 0 ? 0 : kept_before;
 
     const int group = n_heads / n_kv;
     const int kvh = by / head_chunks;
@@ -258,14 +272,16 @@ __global__ __launch_bounds__(kLdsThreads) __attribute__((amdgpu_waves_per_eu(HDT
     // and the window; in a long portion nearly every block): no masks and no branches, one
     // straight run of instructions in which the compiler can place the LDS reads of a product
     // ahead of the arithmetic that precedes it.
-    auto compute_block = [&](int kb, const bf16_t* kbuf, const bf16_t* vbuf, auto inner) {
+    auto compute_block = [&](int kb, const bf16_t* kbuf, const bf16_t* vbuf, auto inner, bool kept_block) {
         constexpr bool INNER = decltype(inner)::value;
         bool use[2];
         floatx4 st[2][NT][2];
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
             const int kh = kb + 32 * h;
-            use[h] = INNER || (kh <= my_last && kh < key_end && kh + 32 > key_begin);  // the same for the whole wave
+            // (the same for the whole wave)
+            use[h] = INNER || (kept_block ? kh < kept_before
+                                          : (kh <= my_last && ((kh < key_end && kh + 32 > key_begin) || kh < kept_in_range)));
             if (!use[h]) continue;
             F16B kf[2][S32];
 #pragma unroll
@@ -294,7 +310,7 @@ __global__ __launch_bounds__(kLdsThreads) __attribute__((amdgpu_waves_per_eu(HDT
         for (int h = 0; h < 2; ++h) {
             if (!use[h]) continue;
             const int kh = kb + 32 * h;
-            const bool full = INNER || (kh >= key_begin && kh + 32 <= key_end && kh + 31 <= pos0 &&
+            const bool full = INNER || (!kept_block && kh >= key_begin && kh + 32 <= key_end && kh + 31 <= pos0 &&
                                         (window <= 0 || kh > pos0 + n_q - 1 - window));
 #pragma unroll
             for (int nt = 0; nt < NT; ++nt) {
@@ -307,8 +323,10 @@ __global__ __launch_bounds__(kLdsThreads) __attribute__((amdgpu_waves_per_eu(HDT
 #pragma unroll
                         for (int r = 0; r < 4; ++r) {
                             const int key = kh + 8 * G + 4 * tt + r;
-                            const bool vis = rvalid[nt] && key >= key_begin && key < key_end && key <= rpos[nt] &&
-                                             (window <= 0 || key > rpos[nt] - window);
+                            const bool in_range = kept_block ? key < kept_before
+                                                             : ((key >= key_begin && key < key_end) || key < kept_in_range);
+                            const bool vis = rvalid[nt] && in_range && key <= rpos[nt] &&
+                                             (window <= 0 || key > rpos[nt] - window || key < keep);
                             sv[h][nt][tt * 4 + r] = vis ? st[h][nt][tt][r] : -INFINITY;
                         }
                 }
@@ -380,18 +398,22 @@ __global__ __launch_bounds__(kLdsThreads) __attribute__((amdgpu_waves_per_eu(HDT
     };
 
     // ---- the blocks: fetch the next one, compute the present one, put the next one into LDS
-    if (wg_begin < wg_end) {
-        fetch(wg_begin);
+    if (walk_first < wg_end) {
+        // (a coordinate before wg_begin: a block of the kept first keys)
+        auto key_of = [&](int u) { return u >= wg_begin ? u : u - walk_first; };
+        fetch(key_of(walk_first));
         stash(0);
         __syncthreads();
         int buf = 0;
-        for (int kb = wg_begin; kb < wg_end; kb += kLdsKeys) {
-            const bool more = kb + kLdsKeys < wg_end;
-            if (more) fetch(kb + kLdsKeys);
-            const bool inner = active && kb >= key_begin && kb + kLdsKeys <= key_end && kb + kLdsKeys - 1 <= pos0 &&
+        for (int u = walk_first; u < wg_end; u += kLdsKeys) {
+            const bool more = u + kLdsKeys < wg_end;
+            if (more) fetch(key_of(u + kLdsKeys));
+            const bool kept_block = u < wg_begin;
+            const int kb = key_of(u);
+            const bool inner = active && !kept_block && kb >= key_begin && kb + kLdsKeys <= key_end && kb + kLdsKeys - 1 <= pos0 &&
                                (window <= 0 || kb > my_last - window);
-            if (inner) compute_block(kb, k_lds[buf], v_lds[buf], std::true_type{});
-            else if (active) compute_block(kb, k_lds[buf], v_lds[buf], std::false_type{});
+            if (inner) compute_block(kb, k_lds[buf], v_lds[buf], std::true_type{}, false);
+            else if (active) compute_block(kb, k_lds[buf], v_lds[buf], std::false_type{}, kept_block);
             if (more) stash(buf ^ 1);
             __syncthreads();
             buf ^= 1;

@@ -79,7 +79,7 @@ class AttentionPlanner:
         return (compute_dtype == torch.bfloat16 and self.head_dim % 16 == 0 and self.head_dim <= 256
                 and page_size % 4 == 0 and (not self.keep_first or self.mfma_keeps_first))
 
-    mfma_keeps_first = False  # whether the matrix-core kernels read an item's kept first keys
+    mfma_keeps_first = True  # whether the matrix-core kernels read an item's kept first keys
 
     def _waves_for(self, keys: int, max_waves: int) -> int:
         """Waves of a workgroup for an item of ``keys`` keys: one per 128 keys, a power of two."""
@@ -427,7 +427,7 @@ class GQAttention(Mixer):
         self.value_dim = head_dim if value_dim is None else int(value_dim)
         self.padded = head_dim if self.value_dim == head_dim else -(-max(head_dim, self.value_dim) // 16) * 16
         if self.padded > 256 or self.value_dim < 1:
-            raise ValueError(f"attention: heads of {head_dim} (values {self.value_dim}) are larger than the kernels take (256)")
+            raise ValueError(f"attention: head_dim {head_dim} (values of {self.value_dim}) is larger than the kernels take (256)")
         if value_mix not in (None, "source", "mixed"):
             raise ValueError(f"attention: value_mix '{value_mix}' is neither 'source' nor 'mixed'")
         if keep_first < 0 or (keep_first and not window):
