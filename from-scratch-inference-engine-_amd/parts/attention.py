@@ -427,7 +427,8 @@ class GQAttention(Mixer):
         self.value_dim = head_dim if value_dim is None else int(value_dim)
         self.padded = head_dim if self.value_dim == head_dim else -(-max(head_dim, self.value_dim) // 16) * 16
         if self.padded > 256 or self.value_dim < 1:
-            raise ValueError(f"attention: head_dim {head_dim} (values of {self.value_dim}) is larger than the kernels take (256)")
+            raise ValueError(f"attention: head_dim {head_dim} is larger than the kernels take (256)" if self.value_dim == head_dim
+                             else f"attention: heads of {head_dim} and values of {self.value_dim} are larger than the kernels take (256)")
         if value_mix not in (None, "source", "mixed"):
             raise ValueError(f"attention: value_mix '{value_mix}' is neither 'source' nor 'mixed'")
         if keep_first < 0 or (keep_first and not window):
