@@ -312,7 +312,7 @@ def design_comparison(args) -> int:
             if times:
                 row["prefill_2048_ms"] = min(times[1:]) * 1e3
                 row["prefill_tok_s"] = 2048 / min(times[1:])
-            for batch in ((8, 64) if "decode" in phases else ()):
+            for batch in ([int(b) for b in args.design_batches.split(",")] if "decode" in phases else ()):
                 caches = [runner.manager.open(f"d{batch}.{i}") for i in range(batch)]
                 for c in caches:
                     runner.step([StepEntry(c, torch.randint(0, vocab, (512,), generator=gen).tolist(), [])])
@@ -360,6 +360,7 @@ def main() -> int:
     ap.add_argument("--no-streamed-copies", action="store_true",
                     help="do not keep the large weights a second time in the order of the matrix instruction's fragments")
     ap.add_argument("--design-sizes", default="2048,4096", help="--workload gilozen | botulorn: widths to run (2048, 4096)")
+    ap.add_argument("--design-batches", default="8,64", help="--workload gilozen | botulorn: decode batches to time (at most 64)")
     ap.add_argument("--design-phases", default="prefill,decode", help="--workload gilozen | botulorn: what to time (for a trace of one phase)")
     ap.add_argument("--workload", choices=["decode", "mixed", "long-prefill", "gilozen", "botulorn"], default="decode",
                     help="decode: the default run.  mixed: --requests prompts of --min-prompt to --max-prompt tokens, "

@@ -30,45 +30,107 @@ __device__ __forceinline__ float normed_turned(const T* __restrict__ x, int j, f
     return j < pairs ? fmaf(a, t.x, -(b * t.y)) : fmaf(a, t.x, b * t.y);
 }
 
-template <typename T>
+// four consecutive values as floats / from floats: one 16-byte (float32) or 8-byte (bfloat16) access
+__device__ __forceinline__ void load4(const float* p, float (&f)[4]) {
+    const float4 v = *reinterpret_cast<const float4*>(p);
+    f[0] = v.x, f[1] = v.y, f[2] = v.z, f[3] = v.w;
+}
+__device__ __forceinline__ void load4(const bf16_t* p, float (&f)[4]) {
+    const uint2 v = *reinterpret_cast<const uint2*>(p);
+    f[0] = __uint_as_float(v.x << 16), f[1] = __uint_as_float(v.x & 0xffff0000u);
+    f[2] = __uint_as_float(v.y << 16), f[3] = __uint_as_float(v.y & 0xffff0000u);
+}
+__device__ __forceinline__ void store4(float* p, const float (&f)[4]) {
+    *reinterpret_cast<float4*>(p) = float4{f[0], f[1], f[2], f[3]};
+}
+__device__ __forceinline__ void store4(bf16_t* p, const float (&f)[4]) {
+    uint2 w;
+    w.x = pack2_bf16(f[0], f[1]);
+    w.y = pack2_bf16(f[2], f[3]);
+    *reinterpret_cast<uint2*>(p) = w;
+}
+
+// VEC: every size, offset and stride is a multiple of 4 and the arrays are 16-byte aligned: a lane takes four
+// neighbouring values (and their four partners of the rotation) with one access each.
+template <typename T, bool VEC>
 __global__ __launch_bounds__(kThreads) void attention_prep_kernel(
     const T* __restrict__ proj, int64_t stride, int q_off, int k_off, int v_off, int g_off, int heads, int kv_heads, int dim,
     int vdim, int D, const float* __restrict__ q_weight, const float* __restrict__ k_weight, float eps, int pairs,
     const float2* __restrict__ cos_sin, const T* __restrict__ v_other, int64_t v_other_stride, const float* __restrict__ mix,
     T* __restrict__ q_out, float* __restrict__ gate, const int32_t* __restrict__ slots, T* __restrict__ k_pool,
-    T* __restrict__ v_pool, int page_size, int64_t pool_slots) {
+    T* __restrict__ v_pool, int page_size, int64_t pool_slots, int values_elsewhere) {
+    // a wave a unit of work: a query head, a key head, a kv head's values, or all gates
     const int t = blockIdx.x;
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63;
+    const int unit = blockIdx.y * (kThreads / 64) + (threadIdx.x >> 6);
     const T* row = proj + static_cast<int64_t>(t) * stride;
-    const float2* cs = cos_sin + static_cast<int64_t>(t) * pairs;
     const int64_t slot = slots ? slots[t] : -1;
     const bool store = k_pool && slot >= 0 && slot < pool_slots;
     const int64_t page = store ? slot / page_size : 0;
     const int off = store ? static_cast<int>(slot - page * page_size) : 0;
-    // a wave a head: the query heads, then the key heads
-    for (int h = wave; h < heads + kv_heads; h += kThreads / 64) {
-        const bool is_q = h < heads;
-        const T* x = row + (is_q ? q_off + h * dim : k_off + (h - heads) * dim);
+    if (unit < heads + kv_heads) {
+        const bool is_q = unit < heads;
+        if (!is_q && !store) return;
+        const T* x = row + (is_q ? q_off + unit * dim : k_off + (unit - heads) * dim);
         const float* w = is_q ? q_weight : k_weight;
-        float scale = 1.f;
-        if (w) {
+        const float2* cs = cos_sin + static_cast<int64_t>(t) * pairs;
+        T* o = is_q ? q_out + (static_cast<int64_t>(t) * heads + unit) * D
+                    : k_pool + ((page * kv_heads + (unit - heads)) * page_size + off) * D;
+        if constexpr (VEC) {
+            // (a head of up to 256 values: one group of four a lane; wider heads go round again)
             float sum = 0.f;
-            for (int j = lane; j < dim; j += 64) sum = fmaf(to_float(x[j]), to_float(x[j]), sum);
-            scale = 1.0f / sqrtf(wave_sum(sum) / static_cast<float>(dim) + eps);
-        }
-        if (is_q) {
-            T* o = q_out + (static_cast<int64_t>(t) * heads + h) * D;
+            if (w) {
+                for (int j = 4 * lane; j < dim; j += 256) {
+                    float a[4];
+                    load4(x + j, a);
+                    sum = fmaf(a[0], a[0], fmaf(a[1], a[1], fmaf(a[2], a[2], fmaf(a[3], a[3], sum))));
+                }
+            }
+            const float scale = w ? 1.0f / sqrtf(wave_sum(sum) / static_cast<float>(dim) + eps) : 1.f;
+            for (int j = 4 * lane; j < D; j += 256) {
+                float a[4] = {0.f, 0.f, 0.f, 0.f};
+                if (j < dim) {
+                    load4(x + j, a);
+                    if (w) {
+                        float ww[4];
+                        load4(w + j, ww);
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) a[i] = (a[i] * scale) * ww[i];
+                    }
+                    if (j < 2 * pairs) {
+                        const bool low = j < pairs;
+                        const int jp = low ? j + pairs : j - pairs;
+                        float b[4], c4[4], s4[4];
+                        load4(x + jp, b);
+                        if (w) {
+                            float ww[4];
+                            load4(w + jp, ww);
+#pragma unroll
+                            for (int i = 0; i < 4; ++i) b[i] = (b[i] * scale) * ww[i];
+                        }
+                        const float2* tp = cs + (low ? j : j - pairs);
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) c4[i] = tp[i].x, s4[i] = tp[i].y;
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) a[i] = low ? fmaf(a[i], c4[i], -(b[i] * s4[i])) : fmaf(a[i], c4[i], b[i] * s4[i]);
+                    }
+                }
+                store4(o + j, a);
+            }
+        } else {
+            float scale = 1.f;
+            if (w) {
+                float sum = 0.f;
+                for (int j = lane; j < dim; j += 64) sum = fmaf(to_float(x[j]), to_float(x[j]), sum);
+                scale = 1.0f / sqrtf(wave_sum(sum) / static_cast<float>(dim) + eps);
+            }
             for (int j = lane; j < D; j += 64) o[j] = from_float<T>(j < dim ? normed_turned(x, j, scale, w, pairs, cs) : 0.f);
-        } else if (store) {
-            const int g = h - heads;
-            T* o = k_pool + ((page * kv_heads + g) * page_size + off) * D;
-            for (int j = lane; j < D; j += 64) o[j] = from_float<T>(j < dim ? normed_turned(x, j, scale, w, pairs, cs) : 0.f);
         }
-    }
-    if (store) {
+    } else if (unit < heads + 2 * kv_heads) {
+        if (!store || values_elsewhere) return;
+        const int g = unit - heads - kv_heads;
         const float lam = (v_other && mix) ? mix[0] : 0.f;
-        for (int e = threadIdx.x; e < kv_heads * D; e += kThreads) {
-            const int g = e / D, j = e - g * D;
+        for (int j = lane; j < D; j += 64) {
             float v = 0.f;
             if (j < vdim) {
                 v = to_float(row[v_off + g * vdim + j]);
@@ -76,22 +138,76 @@ __global__ __launch_bounds__(kThreads) void attention_prep_kernel(
             }
             v_pool[((page * kv_heads + g) * D + j) * page_size + off] = from_float<T>(v);
         }
-    }
-    if (gate) {
-        for (int h = threadIdx.x; h < heads; h += kThreads)
+    } else if (unit == heads + 2 * kv_heads && gate) {
+        for (int h = lane; h < heads; h += 64)
             gate[static_cast<int64_t>(t) * heads + h] = 1.0f / (1.0f + expf(-to_float(row[g_off + h])));
     }
 }
 
-template <typename T>
+// The values of many tokens (a portion of a prompt): a block takes eight consecutive tokens of one kv head, a thread
+// a dimension.  A page of values lies as [dimension][slot], so a token's values are 2-byte pieces a page apart;
+// where the eight tokens fill eight consecutive slots from a multiple of eight (the usual case inside a portion)
+// a thread writes them as one 16-byte piece per dimension.  bfloat16 only (the float32 path writes value by value).
+__global__ __launch_bounds__(kThreads) void attention_prep_values_kernel(
+    const bf16_t* __restrict__ proj, int64_t stride, int v_off, int kv_heads, int vdim, int D,
+    const bf16_t* __restrict__ v_other, int64_t v_other_stride, const float* __restrict__ mix,
+    const int32_t* __restrict__ slots, bf16_t* __restrict__ v_pool, int page_size, int64_t pool_slots, int n_tokens) {
+    const int t0 = blockIdx.x * 8, g = blockIdx.y;
+    const int n = min(8, n_tokens - t0);
+    int64_t slot[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) slot[i] = i < n ? slots[t0 + i] : -1;
+    bool run = n == 8 && slot[0] >= 0 && slot[0] + 7 < pool_slots && (slot[0] & 7) == 0 && (page_size & 7) == 0;
+#pragma unroll
+    for (int i = 1; i < 8; ++i) run = run && slot[i] == slot[0] + i;
+    const float lam = (v_other && mix) ? mix[0] : 0.f;
+    for (int j = threadIdx.x; j < D; j += kThreads) {
+        float v[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            v[i] = 0.f;
+            if (i < n && j < vdim) {
+                v[i] = to_float(proj[static_cast<int64_t>(t0 + i) * stride + v_off + g * vdim + j]);
+                if (v_other) v[i] = fmaf(lam, to_float(v_other[static_cast<int64_t>(t0 + i) * v_other_stride + g * vdim + j]), (1.0f - lam) * v[i]);
+            }
+        }
+        if (run) {
+            const int64_t page = slot[0] / page_size;
+            const int off = static_cast<int>(slot[0] - page * page_size);
+            *reinterpret_cast<uint4*>(v_pool + ((page * kv_heads + g) * D + j) * page_size + off) =
+                uint4{pack2_bf16(v[0], v[1]), pack2_bf16(v[2], v[3]), pack2_bf16(v[4], v[5]), pack2_bf16(v[6], v[7])};
+        } else {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                if (i < n && slot[i] >= 0 && slot[i] < pool_slots) {
+                    const int64_t page = slot[i] / page_size;
+                    const int off = static_cast<int>(slot[i] - page * page_size);
+                    v_pool[((page * kv_heads + g) * D + j) * page_size + off] = from_float<bf16_t>(v[i]);
+                }
+            }
+        }
+    }
+}
+
+// VEC: vdim and D are multiples of 4 and the arrays 16-byte aligned: a thread takes four values of a head
+template <typename T, bool VEC>
 __global__ __launch_bounds__(kThreads) void gate_heads_kernel(const T* __restrict__ x, int D, const float* __restrict__ gate,
                                                               T* __restrict__ y, int heads, int vdim, int64_t total) {
-    const int64_t e = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+    constexpr int N = VEC ? 4 : 1;
+    const int64_t e = (static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x) * N;
     if (e >= total) return;
     const int64_t th = e / vdim;  // token * heads + head
     const int j = static_cast<int>(e - th * vdim);
     const float g = gate ? gate[th] : 1.f;
-    y[e] = from_float<T>(to_float(x[th * D + j]) * g);
+    if constexpr (VEC) {
+        float a[4];
+        load4(x + th * D + j, a);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) a[i] *= g;
+        store4(y + e, a);
+    } else {
+        y[e] = from_float<T>(to_float(x[th * D + j]) * g);
+    }
 }
 
 }  // namespace
@@ -111,14 +227,33 @@ extern "C" int fsie_attention_prep(const void* proj, int64_t stride, int q_off, 
     FSIE_REQUIRE(!v_other || mix, "attention_prep: values to mix in come with their weight");
     FSIE_REQUIRE(dtype == FSIE_F32 || dtype == FSIE_BF16, "attention_prep: unknown dtype %d", dtype);
     if (n_tokens == 0) return 0;
+    const int units = heads + 2 * kv_heads + 1;
+    const dim3 grid(static_cast<unsigned>(n_tokens), static_cast<unsigned>((units + kThreads / 64 - 1) / (kThreads / 64)));
+    const auto mult4 = [](int64_t v) { return (v & 3) == 0; };
+    const auto al16 = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
+    const bool vec = mult4(stride) && mult4(q_off) && mult4(k_off) && mult4(dim) && mult4(D) && mult4(pairs) && al16(proj) &&
+                     al16(q_out) && al16(k_pool) && al16(q_weight) && al16(k_weight) && al16(cos_sin);
 #define FSIE_PREP(T)                                                                                                     \
-    attention_prep_kernel<T><<<n_tokens, kThreads, 0, stream>>>(                                                         \
+    if (vec) FSIE_PREP_V(T, true); else FSIE_PREP_V(T, false)
+#define FSIE_PREP_V(T, V)                                                                                                \
+    attention_prep_kernel<T, V><<<grid, kThreads, 0, stream>>>(                                                      \
         static_cast<const T*>(proj), stride, q_off, k_off, v_off, g_off, heads, kv_heads, dim, vdim, D, q_weight, k_weight, \
         eps, pairs, reinterpret_cast<const float2*>(cos_sin), static_cast<const T*>(v_other), v_other_stride, mix,       \
-        static_cast<T*>(q_out), gate, slots, static_cast<T*>(k_pool), static_cast<T*>(v_pool), page_size, pool_slots)
-    if (dtype == FSIE_F32) FSIE_PREP(float); else FSIE_PREP(bf16_t);
+        static_cast<T*>(q_out), gate, slots, static_cast<T*>(k_pool), static_cast<T*>(v_pool), page_size, pool_slots,   \
+        values_elsewhere)
+    // portions of prompts in bfloat16: the values go through the kernel that writes eight slots at once
+    const int values_elsewhere = (k_pool && dtype == FSIE_BF16 && n_tokens >= 64 && al16(v_pool)) ? 1 : 0;
+    if (dtype == FSIE_F32) { FSIE_PREP(float); } else { FSIE_PREP(bf16_t); }
 #undef FSIE_PREP
+#undef FSIE_PREP_V
     FSIE_CHECK_LAUNCH("attention_prep");
+    if (values_elsewhere) {
+        const dim3 vgrid(static_cast<unsigned>((n_tokens + 7) / 8), static_cast<unsigned>(kv_heads));
+        attention_prep_values_kernel<<<vgrid, kThreads, 0, stream>>>(
+            static_cast<const bf16_t*>(proj), stride, v_off, kv_heads, vdim, D, static_cast<const bf16_t*>(v_other),
+            v_other_stride, mix, slots, static_cast<bf16_t*>(v_pool), page_size, pool_slots, n_tokens);
+        FSIE_CHECK_LAUNCH("attention_prep_values");
+    }
     return 0;
 }
 
@@ -129,13 +264,16 @@ extern "C" int fsie_gate_heads(const void* x, int D, const float* gate, void* y,
     FSIE_REQUIRE(dtype == FSIE_F32 || dtype == FSIE_BF16, "gate_heads: unknown dtype %d", dtype);
     const int64_t total = static_cast<int64_t>(n_tokens) * heads * vdim;
     if (total == 0) return 0;
-    const unsigned grid = static_cast<unsigned>(ceil_div64(total, kThreads));
-    if (dtype == FSIE_F32)
-        gate_heads_kernel<float><<<grid, kThreads, 0, stream>>>(static_cast<const float*>(x), D, gate, static_cast<float*>(y),
-                                                                heads, vdim, total);
-    else
-        gate_heads_kernel<bf16_t><<<grid, kThreads, 0, stream>>>(static_cast<const bf16_t*>(x), D, gate, static_cast<bf16_t*>(y),
-                                                                 heads, vdim, total);
+    const bool vec = vdim % 4 == 0 && D % 4 == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0 && (reinterpret_cast<uintptr_t>(y) & 15) == 0;
+    const unsigned grid = static_cast<unsigned>(ceil_div64(vec ? total / 4 : total, kThreads));
+#define FSIE_GATE(T, V) \
+    gate_heads_kernel<T, V><<<grid, kThreads, 0, stream>>>(static_cast<const T*>(x), D, gate, static_cast<T*>(y), heads, vdim, total)
+    if (dtype == FSIE_F32) {
+        if (vec) FSIE_GATE(float, true); else FSIE_GATE(float, false);
+    } else {
+        if (vec) FSIE_GATE(bf16_t, true); else FSIE_GATE(bf16_t, false);
+    }
+#undef FSIE_GATE
     FSIE_CHECK_LAUNCH("gate_heads");
     return 0;
 }

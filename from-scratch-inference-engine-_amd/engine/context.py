@@ -77,6 +77,9 @@ class HostBatch:
         ) if entries else np.zeros(0, np.int32)
         self.want_rows = np.asarray([self.q_starts[i] + w for i, e in enumerate(entries) for w in e.want],
                                     dtype=np.int32)
+        # the request (index in the step) of every token
+        self.token_seqs = np.repeat(np.arange(self.n_seqs, dtype=np.int64), self.q_lens) if entries else np.zeros(0, np.int64)
+        self.memo = {}  # what a planner computes once for a step and asks for twice (the graph's shape, then the plan)
 
 
 class _Packer:
@@ -211,19 +214,18 @@ def build_context(entries: Sequence[StepEntry], manager: CacheManager, planners:
             if max_pages > pad["pages"]:
                 raise RuntimeError("block tables are wider than the captured graph's")
             max_pages = pad["pages"]
-        table = np.full((len(entries), max_pages), -1, dtype=np.int32)
-        slot_map = np.full((host.n_tokens,), -1, dtype=np.int32)
         # the group's own geometry: a position lies in entry pos // tokens_per_entry, an entry in page
-        # entry // entries_per_page
+        # entry // entries_per_page.  All requests at once (a decode step of many requests is host time
+        # above all): the tables' page ids in one pass, then array arithmetic
         per_entry, ps = manager.tokens_per_entry[g], manager.entries_per_page[g]
-        for s, e in enumerate(entries):
-            # page ids become units of the pool: unit 0 is the null page, page p is unit p + 1
-            pages = np.asarray(e.cache.tables[g], dtype=np.int32)
-            pages = np.where(pages >= 0, pages + 1, -1)
-            table[s, :pages.size] = pages
-            entry = host.positions[host.q_starts[s]:host.q_starts[s + 1]] // per_entry
-            page_of = pages[entry // ps]
-            slot_map[host.q_starts[s]:host.q_starts[s + 1]] = np.where(page_of >= 0, page_of * ps + entry % ps, -1)
+        lens = np.fromiter((len(e.cache.tables[g]) for e in entries), dtype=np.int64, count=len(entries))
+        flat = np.fromiter((p for e in entries for p in e.cache.tables[g]), dtype=np.int32, count=int(lens.sum()))
+        table = np.full((len(entries), max_pages), -1, dtype=np.int32)
+        # page ids become units of the pool: unit 0 is the null page, page p is unit p + 1
+        table[np.arange(max_pages)[None, :] < lens[:, None]] = np.where(flat >= 0, flat + 1, -1)
+        entry = host.positions // per_entry
+        page_of = table[host.token_seqs, entry // ps]
+        slot_map = np.where(page_of >= 0, page_of * ps + entry % ps, -1).astype(np.int32)
         group_idx.append((pk.add(table), pk.add(slot_map)))
     plan_idx = []
     for planner in planners:

@@ -103,6 +103,15 @@ class AttentionPlanner:
         """Keys per small item in this step.  A workgroup draws only so much from memory, so a step
         with few requests is faster with more, shorter items although they cost a merge, and a full
         device keeps the long ones."""
+        memo = getattr(host, "memo", None)
+        if memo is not None and (self.key, mfma, self.compute_units) in memo:
+            return memo[(self.key, mfma, self.compute_units)]
+        split = self._split_keys(host, mfma)
+        if memo is not None:
+            memo[(self.key, mfma, self.compute_units)] = split
+        return split
+
+    def _split_keys(self, host, mfma: bool) -> int:
         small_tokens, _, longest = self.geometry(mfma)
         units = self.compute_units if self.compute_units is not None else ops.compute_units()
         keys = self._small_keys(host, small_tokens)

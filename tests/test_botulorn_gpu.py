@@ -134,22 +134,25 @@ def test_pair_embedding_over_portions_steps_and_slots(ops, dtype, buckets, mul_p
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("t, page", [(11, 4), (83, 8)])
 @pytest.mark.parametrize("heads, kv, dim, vdim, rot, stretch, norms",
                          [(6, 3, 24, 40, 16, (4.0, 32.0, 8.0, 2.0), True), (4, 4, 64, 16, 64, None, True),
                           (2, 1, 32, 32, 0, None, False), (3, 1, 20, 7, 10, (1.0, 64.0, 4.0, 1.0), True)])
-def test_attention_prep_and_gate(ops, dtype, heads, kv, dim, vdim, rot, stretch, norms):
+def test_attention_prep_and_gate(ops, dtype, t, page, heads, kv, dim, vdim, rot, stretch, norms):
     """The kernel between projection and attention against the plain functions: head norms, the rotation of the
     first ``rot`` values with stretched frequencies, values blended with another layer's, gates; what lands in the
-    pools at the tokens' slots (padded heads, zeros at the end, nothing elsewhere)."""
+    pools at the tokens' slots (padded heads, zeros at the end, nothing elsewhere).  A few tokens at scattered
+    slots, and a portion of a prompt whose values go eight slots at a time where they lie so."""
     from from_scratch_inference_engine_amd.parts.rope import RotaryEncoding
 
-    t, page, eps, lam = 11, 4, 1e-5, 0.35
+    eps, lam = 1e-5, 0.35
     padded = dim if dim == vdim else -(-max(dim, vdim) // 16) * 16
     width = heads * dim + kv * dim + kv * vdim + heads
     proj = rnd((t, width + 3), 1).to(dtype)  # (rows longer than what is used)
     other = rnd((t, kv * vdim + 5), 2).to(dtype)
     qw, kw = (rnd((dim,), 3) + 1.0, rnd((dim,), 4) + 1.0) if norms else (None, None)
-    positions = torch.tensor([0, 1, 2, 500, 501, 7, 8, 9, 10, 1234, 3], dtype=torch.int32)
+    positions = ((torch.arange(t) * 389) % 1500).to(torch.int32)
+    positions[:3] = torch.tensor([0, 1, 2], dtype=torch.int32)
     table = None
     rot_cfg = {"base": 500.0, "dims": rot}
     if stretch is not None:
@@ -158,9 +161,13 @@ def test_attention_prep_and_gate(ops, dtype, heads, kv, dim, vdim, rot, stretch,
         enc = RotaryEncoding(dim, 500.0, rotary_dim=rot, layout="half", stretch=stretch)
         enc.prepare("cuda", dtype)
         table = ops.rope_table(positions.cuda(), enc.inv_freq, enc.magnitude)
-    units = 6
-    slots = torch.tensor([page * 2 + 1, page * 2 + 2, page * 2 + 3, page * 4, page * 4 + 1, -1, page * 1, page * 1 + 1,
-                          page * 1 + 2, page * 5 + 3, page * 1 + 3], dtype=torch.int32)
+    # the first half of the tokens from a slot in the middle of a page, the second half from a page's start
+    # (whole runs of eight slots there), one token without a slot, the last ones in a page of their own
+    half = t // 2 if t < 16 else (t // 2) // 8 * 8  # (a run of eight starts at a token whose number is a multiple of eight)
+    slots = torch.cat([page * 2 + 1 + torch.arange(half), page * (4 + half // page) + torch.arange(t - half)]).to(torch.int32)
+    slots[5] = -1
+    slots[-2:] = slots[-3] + 2 * page + torch.arange(2, dtype=torch.int32)
+    units = int(slots.max()) // page + 2
     k_pool = torch.full((units, kv, page, padded), 7.0, dtype=dtype).cuda()
     v_pool = torch.full((units, kv, padded, page), -9.0, dtype=dtype).cuda()
     k_off, v_off = heads * dim, heads * dim + kv * dim
@@ -410,6 +417,16 @@ CONFIG_C = {"architecture": "Botulorn", "width": 64, "vocab": 97, "norm": {"eps"
 ]}
 
 
+# D: sizes that are multiples of nothing: a width that is no multiple of four, heads of 20 with values of 12 and five
+#    rotated pairs, three query heads a kv head, more kept keys than the window is long, a latent of 50 + 6 values.
+CONFIG_D = {"architecture": "Botulorn", "width": 90, "vocab": 101, "norm": {"eps": 1e-5},
+            "embedding": {"scale": 0.5, "bigram": {"buckets": 4099, "mul_prev": 3, "mul_cur": 65537}}, "layers": [
+    layer("latent_attention", latent(5, 10, 6, 14, 50, 22, 9, rotation(77.0, 6, (3.0, 8.0, 2.0, 1.0))), 50),
+    layer("attention", attention(6, 2, 20, 12, 4, 10, rotation(1000.0, 10), v_mix=True), None),
+    layer("attention", attention(2, 2, 28, 12, 64, 2, rotation(1000.0, 0), v_mix=True), 34),
+]}
+
+
 def botulorn_tensors(cfg, seed):
     g = torch.Generator().manual_seed(seed)
     w = cfg["width"]
@@ -448,7 +465,7 @@ def botulorn_tensors(cfg, seed):
 def models(tmp_path_factory):
     root = tmp_path_factory.mktemp("botulorn")
     out = {}
-    for name, cfg in (("A", CONFIG_A), ("B", CONFIG_B), ("C", CONFIG_C)):
+    for name, cfg in (("A", CONFIG_A), ("B", CONFIG_B), ("C", CONFIG_C), ("D", CONFIG_D)):
         d = helpers.make_model_dir(root / name, cfg, 0, tensors=botulorn_tensors(cfg, seed=ord(name)))
         out[name] = (d, plain.read_config(d), plain.read_weights(d))
     return out
@@ -524,7 +541,7 @@ def test_the_plain_model_feels_every_mechanism(models):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B", "C"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
 def test_model_whole_in_portions_decoded_and_batched(models, name, dtype):
     """The same requests whole, token by token (through the captured decode graphs, far enough that every window
     passes over decoded tokens), in portions down to two tokens and one, and in batches of unequal requests that
