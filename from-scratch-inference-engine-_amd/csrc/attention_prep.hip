@@ -50,74 +50,96 @@ __device__ __forceinline__ void store4(bf16_t* p, const float (&f)[4]) {
     *reinterpret_cast<uint2*>(p) = w;
 }
 
-// VEC: every size, offset and stride is a multiple of 4 and the arrays are 16-byte aligned: a lane takes four
-// neighbouring values (and their four partners of the rotation) with one access each.
-template <typename T, bool VEC>
+// VEC: every size, offset and stride is a multiple of 4, heads are at most 256 values and the arrays are 16-byte
+// aligned: a lane takes four neighbouring values with one access.  HPW: units of work a wave takes one after the
+// other (a query head, a key head, a kv head's values, or all gates, in this order); with several, everything they
+// need from memory is asked for before the first reduction, so that a wave's one wait for memory serves them all
+// (portions of prompts: the kernel is made of that wait).
+// With VEC a head takes L = 16, 32 or 64 lanes (four values a lane, L the smallest that holds D), so a wave's pass
+// takes 64 / L heads side by side and its accesses stay wide for small heads.  The workgroups after the first
+// `head_blocks` take the values and the gates, a wave a unit.
+template <typename T, bool VEC, int HPW>
 __global__ __launch_bounds__(kThreads) void attention_prep_kernel(
     const T* __restrict__ proj, int64_t stride, int q_off, int k_off, int v_off, int g_off, int heads, int kv_heads, int dim,
     int vdim, int D, const float* __restrict__ q_weight, const float* __restrict__ k_weight, float eps, int pairs,
     const float2* __restrict__ cos_sin, const T* __restrict__ v_other, int64_t v_other_stride, const float* __restrict__ mix,
     T* __restrict__ q_out, float* __restrict__ gate, const int32_t* __restrict__ slots, T* __restrict__ k_pool,
-    T* __restrict__ v_pool, int page_size, int64_t pool_slots, int values_elsewhere) {
-    // a wave a unit of work: a query head, a key head, a kv head's values, or all gates
+    T* __restrict__ v_pool, int page_size, int64_t pool_slots, int values_elsewhere, int L, int head_blocks) {
     const int t = blockIdx.x;
     const int lane = threadIdx.x & 63;
-    const int unit = blockIdx.y * (kThreads / 64) + (threadIdx.x >> 6);
+    const int side = 64 / L;  // heads side by side in a pass
+    const bool tail = static_cast<int>(blockIdx.y) >= head_blocks;
+    const int unit0 = (blockIdx.y * (kThreads / 64) + (threadIdx.x >> 6)) * HPW * side;
     const T* row = proj + static_cast<int64_t>(t) * stride;
     const int64_t slot = slots ? slots[t] : -1;
     const bool store = k_pool && slot >= 0 && slot < pool_slots;
     const int64_t page = store ? slot / page_size : 0;
     const int off = store ? static_cast<int>(slot - page * page_size) : 0;
-    if (unit < heads + kv_heads) {
-        const bool is_q = unit < heads;
-        if (!is_q && !store) return;
-        const T* x = row + (is_q ? q_off + unit * dim : k_off + (unit - heads) * dim);
-        const float* w = is_q ? q_weight : k_weight;
-        const float2* cs = cos_sin + static_cast<int64_t>(t) * pairs;
-        T* o = is_q ? q_out + (static_cast<int64_t>(t) * heads + unit) * D
-                    : k_pool + ((page * kv_heads + (unit - heads)) * page_size + off) * D;
-        if constexpr (VEC) {
-            // (a head of up to 256 values: one group of four a lane; wider heads go round again)
-            float sum = 0.f;
-            if (w) {
-                for (int j = 4 * lane; j < dim; j += 256) {
-                    float a[4];
-                    load4(x + j, a);
-                    sum = fmaf(a[0], a[0], fmaf(a[1], a[1], fmaf(a[2], a[2], fmaf(a[3], a[3], sum))));
-                }
+    const float2* cs = cos_sin + static_cast<int64_t>(t) * pairs;
+    const int n_heads_all = heads + kv_heads;
+    // where head `unit` is read from, which weight it takes and where it goes (null: nowhere)
+    auto source = [&](int unit) { return row + (unit < heads ? q_off + unit * dim : k_off + (unit - heads) * dim); };
+    auto weight = [&](int unit) { return unit < heads ? q_weight : k_weight; };
+    auto target = [&](int unit) -> T* {
+        if (unit < heads) return q_out + (static_cast<int64_t>(t) * heads + unit) * D;
+        return store ? k_pool + ((page * kv_heads + (unit - heads)) * page_size + off) * D : nullptr;
+    };
+    if constexpr (VEC) {
+        // The partner values of the rotation come from the lane that holds them, already normed, through a lane exchange.
+        const int l = lane & (L - 1), mine = lane / L;
+        const int j = 4 * l;
+        const bool in = j < dim, turned = j < 2 * pairs, low = j < pairs;
+        float a[HPW][4], ww[HPW][4], c4[4] = {1.f, 1.f, 1.f, 1.f}, s4[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int u = 0; u < HPW; ++u) {
+            const int unit = unit0 + u * side + mine;
+            const bool live = !tail && unit < n_heads_all && in;
+            const float* w = unit < n_heads_all ? weight(unit) : nullptr;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) a[u][i] = 0.f, ww[u][i] = 1.f;
+            if (live) load4(source(unit) + j, a[u]);
+            if (live && w) load4(w + j, ww[u]);
+        }
+        if (turned && !tail && unit0 < n_heads_all) {
+            const float2* tp = cs + (low ? j : j - pairs);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) c4[i] = tp[i].x, s4[i] = tp[i].y;
+        }
+        const int partner = (lane & ~(L - 1)) | ((low ? l + (pairs >> 2) : l - (pairs >> 2)) & (L - 1));
+#pragma unroll
+        for (int u = 0; u < HPW; ++u) {
+            if (tail || unit0 + u * side >= n_heads_all) break;  // (the same for the whole wave)
+            const int unit = unit0 + u * side + mine;
+            const bool head = unit < n_heads_all;
+            const bool normed = head && weight(unit) != nullptr;
+            float scale = 1.f;
+            if (q_weight || k_weight) {  // (the same for the whole wave; a head without a weight drops the result)
+                float sum = fmaf(a[u][0], a[u][0], fmaf(a[u][1], a[u][1], fmaf(a[u][2], a[u][2], a[u][3] * a[u][3])));
+                for (int o = L >> 1; o > 0; o >>= 1) sum += __shfl_xor(sum, o, FSIE_WAVE);
+                scale = 1.0f / sqrtf(sum / static_cast<float>(dim) + eps);
             }
-            const float scale = w ? 1.0f / sqrtf(wave_sum(sum) / static_cast<float>(dim) + eps) : 1.f;
-            for (int j = 4 * lane; j < D; j += 256) {
-                float a[4] = {0.f, 0.f, 0.f, 0.f};
-                if (j < dim) {
-                    load4(x + j, a);
-                    if (w) {
-                        float ww[4];
-                        load4(w + j, ww);
+            float b[4];
 #pragma unroll
-                        for (int i = 0; i < 4; ++i) a[i] = (a[i] * scale) * ww[i];
-                    }
-                    if (j < 2 * pairs) {
-                        const bool low = j < pairs;
-                        const int jp = low ? j + pairs : j - pairs;
-                        float b[4], c4[4], s4[4];
-                        load4(x + jp, b);
-                        if (w) {
-                            float ww[4];
-                            load4(w + jp, ww);
-#pragma unroll
-                            for (int i = 0; i < 4; ++i) b[i] = (b[i] * scale) * ww[i];
-                        }
-                        const float2* tp = cs + (low ? j : j - pairs);
-#pragma unroll
-                        for (int i = 0; i < 4; ++i) c4[i] = tp[i].x, s4[i] = tp[i].y;
-#pragma unroll
-                        for (int i = 0; i < 4; ++i) a[i] = low ? fmaf(a[i], c4[i], -(b[i] * s4[i])) : fmaf(a[i], c4[i], b[i] * s4[i]);
-                    }
-                }
-                store4(o + j, a);
+            for (int i = 0; i < 4; ++i) {
+                a[u][i] = normed ? (a[u][i] * scale) * ww[u][i] : a[u][i];
+                b[i] = __shfl(a[u][i], partner, FSIE_WAVE);
             }
-        } else {
+            if (turned) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    a[u][i] = low ? fmaf(a[u][i], c4[i], -(b[i] * s4[i])) : fmaf(a[u][i], c4[i], b[i] * s4[i]);
+            }
+            T* o = head ? target(unit) : nullptr;
+            if (o && j < D) store4(o + j, a[u]);
+        }
+    } else {
+        for (int u = 0; u < HPW && !tail; ++u) {
+            const int unit = unit0 + u;
+            if (unit >= n_heads_all) break;
+            T* o = target(unit);
+            if (!o) continue;
+            const T* x = source(unit);
+            const float* w = weight(unit);
             float scale = 1.f;
             if (w) {
                 float sum = 0.f;
@@ -126,21 +148,25 @@ __global__ __launch_bounds__(kThreads) void attention_prep_kernel(
             }
             for (int j = lane; j < D; j += 64) o[j] = from_float<T>(j < dim ? normed_turned(x, j, scale, w, pairs, cs) : 0.f);
         }
-    } else if (unit < heads + 2 * kv_heads) {
-        if (!store || values_elsewhere) return;
-        const int g = unit - heads - kv_heads;
-        const float lam = (v_other && mix) ? mix[0] : 0.f;
-        for (int j = lane; j < D; j += 64) {
-            float v = 0.f;
-            if (j < vdim) {
-                v = to_float(row[v_off + g * vdim + j]);
-                if (v_other) v = fmaf(lam, to_float(v_other[static_cast<int64_t>(t) * v_other_stride + g * vdim + j]), (1.0f - lam) * v);
+    }
+    if (tail) {
+        const int unit = n_heads_all + (blockIdx.y - head_blocks) * (kThreads / 64) + (threadIdx.x >> 6);
+        if (unit < heads + 2 * kv_heads) {
+            if (!store || values_elsewhere) return;
+            const int g = unit - n_heads_all;
+            const float lam = (v_other && mix) ? mix[0] : 0.f;
+            for (int j = lane; j < D; j += 64) {
+                float v = 0.f;
+                if (j < vdim) {
+                    v = to_float(row[v_off + g * vdim + j]);
+                    if (v_other) v = fmaf(lam, to_float(v_other[static_cast<int64_t>(t) * v_other_stride + g * vdim + j]), (1.0f - lam) * v);
+                }
+                v_pool[((page * kv_heads + g) * D + j) * page_size + off] = from_float<T>(v);
             }
-            v_pool[((page * kv_heads + g) * D + j) * page_size + off] = from_float<T>(v);
+        } else if (unit == heads + 2 * kv_heads && gate) {
+            for (int h = lane; h < heads; h += 64)
+                gate[static_cast<int64_t>(t) * heads + h] = 1.0f / (1.0f + expf(-to_float(row[g_off + h])));
         }
-    } else if (unit == heads + 2 * kv_heads && gate) {
-        for (int h = lane; h < heads; h += 64)
-            gate[static_cast<int64_t>(t) * heads + h] = 1.0f / (1.0f + expf(-to_float(row[g_off + h])));
     }
 }
 
@@ -161,7 +187,7 @@ __global__ __launch_bounds__(kThreads) void attention_prep_values_kernel(
 #pragma unroll
     for (int i = 1; i < 8; ++i) run = run && slot[i] == slot[0] + i;
     const float lam = (v_other && mix) ? mix[0] : 0.f;
-    for (int j = threadIdx.x; j < D; j += kThreads) {
+    for (int j = threadIdx.x; j < D; j += blockDim.x) {
         float v[8];
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
@@ -227,29 +253,40 @@ extern "C" int fsie_attention_prep(const void* proj, int64_t stride, int q_off, 
     FSIE_REQUIRE(!v_other || mix, "attention_prep: values to mix in come with their weight");
     FSIE_REQUIRE(dtype == FSIE_F32 || dtype == FSIE_BF16, "attention_prep: unknown dtype %d", dtype);
     if (n_tokens == 0) return 0;
-    const int units = heads + 2 * kv_heads + 1;
-    const dim3 grid(static_cast<unsigned>(n_tokens), static_cast<unsigned>((units + kThreads / 64 - 1) / (kThreads / 64)));
     const auto mult4 = [](int64_t v) { return (v & 3) == 0; };
     const auto al16 = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
-    const bool vec = mult4(stride) && mult4(q_off) && mult4(k_off) && mult4(dim) && mult4(D) && mult4(pairs) && al16(proj) &&
+    const bool vec = D <= 256 && mult4(stride) && mult4(q_off) && mult4(k_off) && mult4(dim) && mult4(D) && mult4(pairs) && al16(proj) &&
                      al16(q_out) && al16(k_pool) && al16(q_weight) && al16(k_weight) && al16(cos_sin);
-#define FSIE_PREP(T)                                                                                                     \
-    if (vec) FSIE_PREP_V(T, true); else FSIE_PREP_V(T, false)
-#define FSIE_PREP_V(T, V)                                                                                                \
-    attention_prep_kernel<T, V><<<grid, kThreads, 0, stream>>>(                                                      \
+    // portions of prompts in bfloat16: the values go through the kernel that writes eight slots at once
+    const int values_elsewhere = (k_pool && dtype == FSIE_BF16 && n_tokens >= 64 && al16(v_pool)) ? 1 : 0;
+    // many tokens: four units a wave (see the kernel); few: one, so that a decode step has waves enough
+    const int hpw = n_tokens >= 64 ? 4 : 1;
+    const int lanes = vec ? (D <= 64 ? 16 : (D <= 128 ? 32 : 64)) : 64;  // lanes a head
+    const int per_block = (kThreads / 64) * hpw * (64 / lanes);
+    const int head_blocks = (heads + kv_heads + per_block - 1) / per_block;
+    // behind the heads: a unit a kv head's values, then one for the gates (with the values written elsewhere and
+    // gates to make, the values' waves leave at once)
+    const int tail_units = gate ? kv_heads + 1 : (values_elsewhere || !k_pool ? 0 : kv_heads);
+    const int tail_blocks = (tail_units + kThreads / 64 - 1) / (kThreads / 64);
+    const dim3 grid(static_cast<unsigned>(n_tokens), static_cast<unsigned>(head_blocks + tail_blocks));
+#define FSIE_PREP_H(T, V, H)                                                                                             \
+    attention_prep_kernel<T, V, H><<<grid, kThreads, 0, stream>>>(                                                       \
         static_cast<const T*>(proj), stride, q_off, k_off, v_off, g_off, heads, kv_heads, dim, vdim, D, q_weight, k_weight, \
         eps, pairs, reinterpret_cast<const float2*>(cos_sin), static_cast<const T*>(v_other), v_other_stride, mix,       \
         static_cast<T*>(q_out), gate, slots, static_cast<T*>(k_pool), static_cast<T*>(v_pool), page_size, pool_slots,   \
-        values_elsewhere)
-    // portions of prompts in bfloat16: the values go through the kernel that writes eight slots at once
-    const int values_elsewhere = (k_pool && dtype == FSIE_BF16 && n_tokens >= 64 && al16(v_pool)) ? 1 : 0;
-    if (dtype == FSIE_F32) { FSIE_PREP(float); } else { FSIE_PREP(bf16_t); }
+        values_elsewhere, lanes, head_blocks)
+#define FSIE_PREP_V(T, V) \
+    if (hpw == 4) FSIE_PREP_H(T, V, 4); else FSIE_PREP_H(T, V, 1)
+#define FSIE_PREP(T) \
+    if (vec) { FSIE_PREP_V(T, true); } else { FSIE_PREP_V(T, false); }
+    if (dtype == FSIE_F32) { FSIE_PREP(float) } else { FSIE_PREP(bf16_t) }
 #undef FSIE_PREP
 #undef FSIE_PREP_V
+#undef FSIE_PREP_H
     FSIE_CHECK_LAUNCH("attention_prep");
     if (values_elsewhere) {
         const dim3 vgrid(static_cast<unsigned>((n_tokens + 7) / 8), static_cast<unsigned>(kv_heads));
-        attention_prep_values_kernel<<<vgrid, kThreads, 0, stream>>>(
+        attention_prep_values_kernel<<<vgrid, D <= 64 ? 64 : (D <= 128 ? 128 : kThreads), 0, stream>>>(
             static_cast<const bf16_t*>(proj), stride, v_off, kv_heads, vdim, D, static_cast<const bf16_t*>(v_other),
             v_other_stride, mix, slots, static_cast<bf16_t*>(v_pool), page_size, pool_slots, n_tokens);
         FSIE_CHECK_LAUNCH("attention_prep_values");
