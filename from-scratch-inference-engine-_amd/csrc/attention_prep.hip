@@ -17,6 +17,8 @@
 namespace {
 
 constexpr int kThreads = 256;
+// steps of this many tokens and more are taken to be portions of prompts (consecutive slots), fewer a decode batch
+constexpr int kPortionTokens = 256;
 
 // value j of a head's run x[0 .. dim) after norm (factor `scale`, weight w or none) and rotation
 template <typename T>
@@ -258,9 +260,9 @@ extern "C" int fsie_attention_prep(const void* proj, int64_t stride, int q_off, 
     const bool vec = D <= 256 && mult4(stride) && mult4(q_off) && mult4(k_off) && mult4(dim) && mult4(D) && mult4(pairs) && al16(proj) &&
                      al16(q_out) && al16(k_pool) && al16(q_weight) && al16(k_weight) && al16(cos_sin);
     // portions of prompts in bfloat16: the values go through the kernel that writes eight slots at once
-    const int values_elsewhere = (k_pool && dtype == FSIE_BF16 && n_tokens >= 64 && al16(v_pool)) ? 1 : 0;
+    const int values_elsewhere = (k_pool && dtype == FSIE_BF16 && n_tokens >= kPortionTokens && al16(v_pool)) ? 1 : 0;
     // many tokens: four units a wave (see the kernel); few: one, so that a decode step has waves enough
-    const int hpw = n_tokens >= 64 ? 4 : 1;
+    const int hpw = n_tokens >= kPortionTokens ? 4 : 1;
     const int lanes = vec ? (D <= 64 ? 16 : (D <= 128 ? 32 : 64)) : 64;  // lanes a head
     const int per_block = (kThreads / 64) * hpw * (64 / lanes);
     const int head_blocks = (heads + kv_heads + per_block - 1) / per_block;

@@ -134,7 +134,7 @@ def test_pair_embedding_over_portions_steps_and_slots(ops, dtype, buckets, mul_p
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("t, page", [(11, 4), (83, 8)])
+@pytest.mark.parametrize("t, page", [(11, 4), (83, 8), (299, 8)])
 @pytest.mark.parametrize("heads, kv, dim, vdim, rot, stretch, norms",
                          [(6, 3, 24, 40, 16, (4.0, 32.0, 8.0, 2.0), True), (4, 4, 64, 16, 64, None, True),
                           (2, 1, 32, 32, 0, None, False), (3, 1, 20, 7, 10, (1.0, 64.0, 4.0, 1.0), True)])
