@@ -254,18 +254,18 @@ def gilozen_shape(width: int, ff: int, layers: int, vocab: int) -> dict:
 
 def botulorn_shape(width: int, ff: int, layers: int, vocab: int) -> dict:
     """A Botulorn configuration of real layer sizes: attention through a latent and grouped-query attention in
-    turn (windows of 1,024 positions, the latter keeping a request's first four), every layer with a gated
+    turn (windows of 1,024 positions, the latter keeping a request's first eight), every layer with a gated
     feed-forward beside its mixer."""
     heads = width // 128
-    stretch = {"factor": 8.0, "original": 1024, "fast": 32.0, "slow": 1.0}
+    stretch = {"factor": 4.0, "original": 2048, "fast": 16.0, "slow": 2.0}
     latent = {"heads": heads, "dim": 64, "rot_dim": 64, "vdim": 128, "kv_rank": 192, "q_rank": width // 2 + 256,
               "scale": 128 ** -0.5, "mask": {"size": 1024}, "rot": {"base": 500000.0, "dims": 64, "scaling": stretch}}
     gqa = {"heads": heads, "kv_heads": max(1, width // 512), "dim": 128, "vdim": 128, "scale": 128 ** -0.5, "v_mix": True,
-           "mask": {"size": 1024, "keep_first": 4}, "rot": {"base": 500000.0, "dims": 64, "scaling": stretch}}
+           "mask": {"size": 1024, "keep_first": 8}, "rot": {"base": 500000.0, "dims": 64, "scaling": stretch}}
     out = [{"type": "latent_attention" if i % 2 == 0 else "attention", "mixer": dict(latent if i % 2 == 0 else gqa),
             "mlp": {"kind": "dense", "ff": ff}} for i in range(layers)]
     return {"architecture": "Botulorn", "width": width, "vocab": vocab, "norm": {"eps": 1e-5},
-            "embedding": {"scale": width ** 0.5, "bigram": {"buckets": 65521, "mul_prev": 1000003, "mul_cur": 7}},
+            "embedding": {"scale": 12.0, "bigram": {"buckets": 65521, "mul_prev": 1000003, "mul_cur": 31}},
             "layers": out}
 
 

@@ -63,7 +63,7 @@ def test_configuration_refuses(edit, message):
         parse_config(raw)
 
 
-@pytest.mark.parametrize("rot", [{"base": 10000.0, "dims": 64, "scaling": {"factor": 8.0, "original": 512, "fast": 32.0, "slow": 1.0}},
+@pytest.mark.parametrize("rot", [{"base": 20000.0, "dims": 48, "scaling": {"factor": 6.0, "original": 256, "fast": 24.0, "slow": 0.5}},
                                  {"base": 500.0, "dims": 16, "scaling": {"factor": 4.0, "original": 32, "fast": 8.0, "slow": 2.0}},
                                  {"base": 1e6, "dims": 24, "scaling": {"factor": 1.0, "original": 100, "fast": 3.0, "slow": 3.0}},
                                  {"base": 100.0, "dims": 6}])

@@ -282,7 +282,7 @@ def kernel_families():
 
 
 @pytest.mark.parametrize("family", range(3))
-@pytest.mark.parametrize("heads, kv, hd, window, keep, page", [(4, 2, 64, 96, 4, 16), (6, 1, 32, 40, 9, 8), (2, 2, 48, 17, 1, 16),
+@pytest.mark.parametrize("heads, kv, hd, window, keep, page", [(4, 2, 64, 80, 3, 16), (6, 1, 32, 40, 9, 8), (2, 2, 48, 17, 1, 16),
                                                                (8, 2, 128, 200, 35, 16)])
 def test_attention_that_keeps_first_keys_on_every_kernel(ops, family, heads, kv, hd, window, keep, page):
     """Random queries and keys: decodes far past the window (cut into items and merged, the kept keys an item of
