@@ -58,6 +58,7 @@ class CacheManager:
         if len(num_pages) != len(self.groups):
             raise ValueError("CacheManager: num_pages must match the number of groups")
         self.allocators = [PageAllocator(int(n)) for n in num_pages]
+        self._page_tokens = [e * t for e, t in zip(self.entries_per_page, self.tokens_per_entry)]  # positions a page of each group holds
         self.max_requests = int(max_requests)
         self._free_slots = list(range(self.max_requests - 1, -1, -1))
         self._live: Dict[Hashable, RequestCache] = {}
@@ -134,7 +135,8 @@ class CacheManager:
 
     def new_pages_needed(self, rc: RequestCache, n_tokens: int) -> List[int]:
         """Pages each group must take from its pool to hold ``n_tokens`` more."""
-        return [max(0, self.pages_for(rc.length + n_tokens, g) - len(t)) for g, t in enumerate(rc.tables)]
+        total = rc.length + n_tokens
+        return [max(0, -(-total // per_page) - len(t)) for per_page, t in zip(self._page_tokens, rc.tables)]
 
     def max_pages_held(self, total_tokens: int, portion: int) -> List[int]:
         """Upper bound of pages a request of ``total_tokens`` holds at once per group when it is

@@ -7,6 +7,7 @@ device views of it."""
 from __future__ import annotations
 
 from dataclasses import dataclass, field
+from itertools import chain
 from types import SimpleNamespace
 from typing import Dict, Hashable, List, Optional, Sequence
 
@@ -219,7 +220,7 @@ def build_context(entries: Sequence[StepEntry], manager: CacheManager, planners:
         # above all): the tables' page ids in one pass, then array arithmetic
         per_entry, ps = manager.tokens_per_entry[g], manager.entries_per_page[g]
         lens = np.fromiter((len(e.cache.tables[g]) for e in entries), dtype=np.int64, count=len(entries))
-        flat = np.fromiter((p for e in entries for p in e.cache.tables[g]), dtype=np.int32, count=int(lens.sum()))
+        flat = np.fromiter(chain.from_iterable(e.cache.tables[g] for e in entries), dtype=np.int32, count=int(lens.sum()))
         table = np.full((len(entries), max_pages), -1, dtype=np.int32)
         # page ids become units of the pool: unit 0 is the null page, page p is unit p + 1
         table[np.arange(max_pages)[None, :] < lens[:, None]] = np.where(flat >= 0, flat + 1, -1)
